@@ -1,0 +1,104 @@
+/* C ABI of libomni_moe_hip.so: the OmniMoE forward path on AMD Instinct MI355X (gfx950).
+ *
+ * Plain pointers and sizes only.  Every pointer named "device" is a device address
+ * of a densely packed row-major array.  Every call enqueues its kernels on `stream`
+ * (a hipStream_t passed as void*, NULL = the default stream) and returns without
+ * waiting for the device.  The library allocates no memory: outputs and workspaces
+ * come from the caller (the *_workspace_bytes calls give the sizes).  Inputs are
+ * never written.  It keeps no mutable global state, so calls are re-entrant as long
+ * as their outputs and workspaces are distinct.
+ *
+ * Return value: OMNI_OK (0); a negative OMNI_ERR_* for a rejected argument (nothing
+ * was enqueued); OMNI_ERR_HIP_BASE + hipError_t when the HIP runtime refused a launch.
+ *
+ * Citations are file:line in the reference tree (HKUSTDial/omni-moe).
+ */
+#ifndef OMNI_MOE_HIP_H_
+#define OMNI_MOE_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define OMNI_ABI_VERSION 1
+
+#if defined(__GNUC__)
+#define OMNI_API __attribute__((visibility("default")))
+#else
+#define OMNI_API
+#endif
+
+/* storage dtype of activations / weights / scores */
+#define OMNI_BF16 0
+#define OMNI_F16 1
+#define OMNI_F32 2
+
+#define OMNI_OK 0
+#define OMNI_ERR_NULL (-1)        /* a required pointer is NULL */
+#define OMNI_ERR_SHAPE (-2)       /* a size is negative, misaligned or out of range */
+#define OMNI_ERR_DTYPE (-3)       /* unknown dtype code */
+#define OMNI_ERR_TOPK (-4)        /* num_experts_per_token violates the router contract */
+#define OMNI_ERR_UNSUPPORTED (-5) /* valid request that no kernel here covers */
+#define OMNI_ERR_WORKSPACE (-6)   /* workspace NULL or too small */
+#define OMNI_ERR_HIP_BASE 1000    /* + hipError_t */
+
+/* expert algorithms */
+#define OMNI_EXPERT_ALGO_AUTO 0
+#define OMNI_EXPERT_ALGO_GATHER 1   /* token-resident gather, no schedule needed */
+#define OMNI_EXPERT_ALGO_SEGMENT 2  /* expert-centric segments from omni_schedule */
+
+OMNI_API int32_t omni_abi_version(void);
+OMNI_API const char* omni_error_string(int32_t code);
+
+/* Cartesian-product router selection.
+ * Replaces triton_omni_router_func / _omni_router_forward
+ * (omni_moe/ops/triton/interface.py:32-51, omni_router.py:167-232, kernel :8-95)
+ * including its two torch.topk pre-steps (:186-189).
+ *   logits_x, logits_y : device [num_tokens, num_expert_sqrt], dtype `dtype`
+ *   scores             : device [num_tokens, k], dtype `dtype`, descending
+ *   indices            : device [num_tokens, k] int32, ix*num_expert_sqrt+iy
+ * Contract of utils.py:81-104: 0 <= k <= r*r, k <= 128, k even (else OMNI_ERR_TOPK).
+ * Ties: the lower key index wins inside a half; the lower candidate position
+ * a*k'+b (a, b = ranks in the two halves, k' = min(r,k)) wins among equal sums. */
+OMNI_API int32_t omni_router_select(const void* logits_x, const void* logits_y, void* scores, int32_t* indices,
+                           int64_t num_tokens, int32_t num_expert_sqrt, int32_t num_experts_per_token,
+                           int32_t dtype, void* stream);
+
+/* Expert-centric schedule: counting sort of the (token, expert) pairs by expert id.
+ * Replaces get_scheduling_info's tail part (omni_moe/ops/triton/omni_scheduler.py:48-101).
+ *   indices          : device [num_tokens, k] int32, each in [0, num_experts)
+ *   offsets          : device [num_experts+1] int32; pairs of expert e occupy
+ *                      [offsets[e], offsets[e+1]) of the sorted arrays
+ *   sorted_pair_ids  : device [num_tokens*k] int32, pair id = token*k + slot;
+ *                      inside a segment ascending (stable)
+ *   sorted_token_ids : device [num_tokens*k] int32 (= sorted_pair_ids / k), may be NULL
+ *   workspace        : device, omni_schedule_workspace_bytes() bytes */
+OMNI_API size_t omni_schedule_workspace_bytes(int64_t num_tokens, int32_t num_experts_per_token, int64_t num_experts);
+OMNI_API int32_t omni_schedule(const int32_t* indices, int32_t* offsets, int32_t* sorted_pair_ids,
+                      int32_t* sorted_token_ids, int64_t num_tokens, int32_t num_experts_per_token,
+                      int64_t num_experts, void* workspace, void* stream);
+
+/* Fused atomic-expert forward  y[t] = sum_j silu(<x[t],U[id_tj]>) * g_tj * V[id_tj].
+ * Replaces triton_omni_expert_func / omni_expert_forward
+ * (interface.py:54-72, omni_expert.py:920-992 with kernels :8-87 and :90-168).
+ *   x [T,H], up_weight [N,H], down_weight [N,H], routing_weights [T,k] : dtype `dtype`
+ *   indices [T,k] int32 in [0,N) (duplicates inside a token add; not range-checked,
+ *   as in the reference); y [T,H] dtype `dtype`, fully overwritten.
+ * H*sizeof(elem) must be a multiple of 16.  Sums are fp32, one rounding at the end.
+ *   algo      : OMNI_EXPERT_ALGO_*
+ *   workspace : omni_expert_workspace_bytes() bytes (0 for GATHER: may be NULL) */
+OMNI_API size_t omni_expert_workspace_bytes(int64_t num_tokens, int32_t hidden_size, int64_t num_experts,
+                                   int32_t num_experts_per_token, int32_t dtype, int32_t algo);
+OMNI_API int32_t omni_expert_fwd(const void* x, const void* up_weight, const void* down_weight,
+                        const void* routing_weights, const int32_t* indices, void* y,
+                        int64_t num_tokens, int32_t hidden_size, int64_t num_experts,
+                        int32_t num_experts_per_token, int32_t dtype, int32_t algo,
+                        void* workspace, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* OMNI_MOE_HIP_H_ */

@@ -1,0 +1,79 @@
+// Device-side helpers shared by the gfx950 kernels of the OmniMoE forward path.
+// Wave size is 64 throughout; nothing here is written for any other target.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace omni {
+
+constexpr int kWave = 64;
+
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
+// Storage dtypes of the operator API (values match include/omni_moe_hip.h).
+enum : int { kBF16 = 0, kF16 = 1, kF32 = 2 };
+
+// ---- scalar conversions ----------------------------------------------------
+__device__ __forceinline__ float bf16_bits_to_f32(uint16_t b) { return __uint_as_float(uint32_t(b) << 16); }
+__device__ __forceinline__ float bf16_lo(uint32_t p) { return __uint_as_float(p << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t p) { return __uint_as_float(p & 0xffff0000u); }
+
+// two floats -> packed bf16 pair, round-to-nearest-even (v_cvt_pk_bf16_f32)
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+  f32x2_t f = {lo, hi};
+  bf16x2_t r = __builtin_convertvector(f, bf16x2_t);
+  return __builtin_bit_cast(uint32_t, r);
+}
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) { return uint16_t(pack_bf16(f, 0.f) & 0xffffu); }
+__device__ __forceinline__ float round_to_bf16(float f) { return bf16_lo(pack_bf16(f, 0.f)); }
+
+__device__ __forceinline__ float f16_bits_to_f32(uint16_t b) { return float(__builtin_bit_cast(_Float16, b)); }
+__device__ __forceinline__ uint16_t f32_to_f16_bits(float f) { return __builtin_bit_cast(uint16_t, _Float16(f)); }
+__device__ __forceinline__ uint32_t pack_f16(float lo, float hi) {
+  return uint32_t(f32_to_f16_bits(lo)) | (uint32_t(f32_to_f16_bits(hi)) << 16);
+}
+
+// Per-dtype element traits used by the bandwidth-bound kernels.
+template <int DT> struct Elem;
+template <> struct Elem<kBF16> {
+  typedef uint16_t store_t;
+  static __device__ __forceinline__ float load(const void* p, int64_t i) { return bf16_bits_to_f32(((const uint16_t*)p)[i]); }
+  static __device__ __forceinline__ void store(void* p, int64_t i, float v) { ((uint16_t*)p)[i] = f32_to_bf16_bits(v); }
+  static __device__ __forceinline__ float round(float v) { return round_to_bf16(v); }
+};
+template <> struct Elem<kF16> {
+  typedef uint16_t store_t;
+  static __device__ __forceinline__ float load(const void* p, int64_t i) { return f16_bits_to_f32(((const uint16_t*)p)[i]); }
+  static __device__ __forceinline__ void store(void* p, int64_t i, float v) { ((uint16_t*)p)[i] = f32_to_f16_bits(v); }
+  static __device__ __forceinline__ float round(float v) { return float(_Float16(v)); }
+};
+template <> struct Elem<kF32> {
+  typedef float store_t;
+  static __device__ __forceinline__ float load(const void* p, int64_t i) { return ((const float*)p)[i]; }
+  static __device__ __forceinline__ void store(void* p, int64_t i, float v) { ((float*)p)[i] = v; }
+  static __device__ __forceinline__ float round(float v) { return v; }
+};
+
+// ---- wave-level primitives ---------------------------------------------------
+__device__ __forceinline__ int lane_id() { return threadIdx.x & (kWave - 1); }
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int m = kWave / 2; m >= 1; m >>= 1) v += __shfl_xor(v, m, kWave);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int m = kWave / 2; m >= 1; m >>= 1) v = fmaxf(v, __shfl_xor(v, m, kWave));
+  return v;
+}
+
+// x*sigmoid(x) in fp32.  expf keeps full fp32 accuracy; the division is IEEE.
+__device__ __forceinline__ float silu_f32(float x) { return x / (1.0f + __expf(-x)); }
+
+}  // namespace omni

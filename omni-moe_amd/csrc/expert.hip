@@ -1,0 +1,217 @@
+// Fused atomic-expert forward for gfx950:
+//     y[t,:] = sum_j silu(<x[t,:], U[id[t,j],:]>) * g[t,j] * V[id[t,j],:]
+// replacing the reference's schedule + two Triton kernels + fp32 score buffer
+// (omni_moe/ops/triton/omni_expert.py:8-168, 920-992) with one launch.
+//
+// Token-resident gather ("gather" algorithm): one 64-lane wave owns one token.
+// The token's row of x stays in registers (16 B per lane per 1 KiB of row), each
+// selected expert's up row and down row is fetched with one fully coalesced
+// 128-bit load per lane per 1 KiB, the dot product is reduced across the wave,
+// and the gate-weighted down rows accumulate in fp32 registers.  Nothing but y
+// is written: no score buffer, no atomics, and the summation order is fixed
+// (slot 0..k-1), so results are run-to-run identical.
+#include "common.h"
+#include "omni_moe_hip.h"
+
+namespace omni {
+
+template <int DT> struct Row16 {               // what one 16-byte lane load holds
+  static constexpr int kElems = (DT == kF32) ? 4 : 8;
+};
+
+template <int DT>
+__device__ __forceinline__ float dot16(const u32x4_t a, const u32x4_t b, float acc) {
+  if constexpr (DT == kBF16) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t ai = a[i], bi = b[i];     // bit_cast wants a scalar object, not a vector element
+      acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, ai), __builtin_bit_cast(bf16x2_t, bi), acc, false);
+    }
+  } else if constexpr (DT == kF16) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t ai = a[i], bi = b[i];
+      f16x2_t p = __builtin_bit_cast(f16x2_t, ai), q = __builtin_bit_cast(f16x2_t, bi);
+      acc = fmaf(float(p[0]), float(q[0]), acc);
+      acc = fmaf(float(p[1]), float(q[1]), acc);
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc = fmaf(__uint_as_float(a[i]), __uint_as_float(b[i]), acc);
+  }
+  return acc;
+}
+
+// acc[0..kElems) += c * row
+template <int DT>
+__device__ __forceinline__ void axpy16(float c, const u32x4_t v, float* acc) {
+  if constexpr (DT == kBF16) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t vi = v[i];
+      acc[2 * i] = fmaf(c, bf16_lo(vi), acc[2 * i]);
+      acc[2 * i + 1] = fmaf(c, bf16_hi(vi), acc[2 * i + 1]);
+    }
+  } else if constexpr (DT == kF16) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t vi = v[i];
+      f16x2_t p = __builtin_bit_cast(f16x2_t, vi);
+      acc[2 * i] = fmaf(c, float(p[0]), acc[2 * i]);
+      acc[2 * i + 1] = fmaf(c, float(p[1]), acc[2 * i + 1]);
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc[i] = fmaf(c, __uint_as_float(v[i]), acc[i]);
+  }
+}
+
+template <int DT>
+__device__ __forceinline__ u32x4_t pack16(const float* acc) {
+  u32x4_t o;
+  if constexpr (DT == kBF16) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o[i] = pack_bf16(acc[2 * i], acc[2 * i + 1]);
+  } else if constexpr (DT == kF16) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o[i] = pack_f16(acc[2 * i], acc[2 * i + 1]);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o[i] = __float_as_uint(acc[i]);
+  }
+  return o;
+}
+
+constexpr int kTokensPerBlock = 4;   // one wave each
+
+// NCH = 16-byte chunks of a row per lane (row bytes / 1024, rounded up);
+// G   = experts fetched per batch (their 2*G*NCH loads are all in flight at once).
+template <int DT, int NCH, int G>
+__global__ __launch_bounds__(kTokensPerBlock* kWave, 2) void expert_gather_kernel(
+    const uint8_t* __restrict__ x, const uint8_t* __restrict__ up, const uint8_t* __restrict__ down,
+    const void* __restrict__ gates, const int32_t* __restrict__ ids, uint8_t* __restrict__ y,
+    int num_tokens, int hidden, int top_k, uint32_t num_experts) {
+  constexpr int E = Row16<DT>::kElems;
+  const int lane = lane_id();
+  const int t = __builtin_amdgcn_readfirstlane(blockIdx.x * kTokensPerBlock + (threadIdx.x >> 6));
+  if (t >= num_tokens) return;
+  const int64_t row_bytes = int64_t(hidden) * (16 / E);
+
+  bool live[NCH];
+  int64_t off[NCH];                    // byte offset of this lane's chunk c inside a row
+  u32x4_t xr[NCH];
+  float acc[NCH][E];
+#pragma unroll
+  for (int c = 0; c < NCH; ++c) {
+    const int first = (c * kWave + lane) * E;
+    live[c] = first < hidden;
+    off[c] = int64_t(c * kWave + lane) * 16;
+    xr[c] = live[c] ? *(const u32x4_t*)(x + t * row_bytes + off[c]) : u32x4_t{0, 0, 0, 0};
+#pragma unroll
+    for (int i = 0; i < E; ++i) acc[c][i] = 0.f;
+  }
+
+  const int32_t* my_ids = ids + int64_t(t) * top_k;
+  for (int j0 = 0; j0 < top_k; j0 += G) {
+    int e[G];
+    float g[G];
+    bool live_slot[G];
+#pragma unroll
+    for (int i = 0; i < G; ++i) {
+      const int j = min(j0 + i, top_k - 1);          // always a valid slot: no branch around the loads
+      const int id = my_ids[j];
+      const float gate = Elem<DT>::load(gates, int64_t(t) * top_k + j);
+      // a slot past k, or an id outside the table, contributes nothing
+      const bool ok = (j0 + i < top_k) && (uint32_t)id < num_experts;
+      e[i] = ok ? id : 0;
+      g[i] = ok ? gate : 0.f;
+      live_slot[i] = ok;
+    }
+    u32x4_t ur[G][NCH], vr[G][NCH];
+#pragma unroll
+    for (int i = 0; i < G; ++i)
+#pragma unroll
+      for (int c = 0; c < NCH; ++c)
+        ur[i][c] = live[c] ? *(const u32x4_t*)(up + e[i] * row_bytes + off[c]) : u32x4_t{0, 0, 0, 0};
+#pragma unroll
+    for (int i = 0; i < G; ++i)
+#pragma unroll
+      for (int c = 0; c < NCH; ++c)
+        vr[i][c] = live[c] ? *(const u32x4_t*)(down + e[i] * row_bytes + off[c]) : u32x4_t{0, 0, 0, 0};
+
+    float s[G];
+#pragma unroll
+    for (int i = 0; i < G; ++i) {
+      float p = 0.f;
+#pragma unroll
+      for (int c = 0; c < NCH; ++c) p = dot16<DT>(xr[c], ur[i][c], p);
+      s[i] = p;
+    }
+#pragma unroll
+    for (int i = 0; i < G; ++i) s[i] = wave_sum(s[i]);
+#pragma unroll
+    for (int i = 0; i < G; ++i) {
+      const float coef = live_slot[i] ? silu_f32(s[i]) * g[i] : 0.f;
+#pragma unroll
+      for (int c = 0; c < NCH; ++c) axpy16<DT>(coef, vr[i][c], acc[c]);
+    }
+  }
+
+#pragma unroll
+  for (int c = 0; c < NCH; ++c)
+    if (live[c]) *(u32x4_t*)(y + t * row_bytes + off[c]) = pack16<DT>(acc[c]);
+}
+
+template <int DT, int NCH, int G>
+static hipError_t launch_gather(const void* x, const void* up, const void* down, const void* gates,
+                                const int32_t* ids, void* y, int64_t T, int H, int k, int64_t N, hipStream_t s) {
+  if (T == 0) return hipSuccess;
+  dim3 grid((unsigned)((T + kTokensPerBlock - 1) / kTokensPerBlock)), block(kTokensPerBlock * kWave);
+  hipLaunchKernelGGL((expert_gather_kernel<DT, NCH, G>), grid, block, 0, s, (const uint8_t*)x, (const uint8_t*)up,
+                     (const uint8_t*)down, gates, ids, (uint8_t*)y, (int)T, H, k, (uint32_t)N);
+  return hipGetLastError();
+}
+
+template <int DT>
+static int expert_gather_dispatch(const void* x, const void* up, const void* down, const void* gates,
+                                  const int32_t* ids, void* y, int64_t T, int H, int k, int64_t N, hipStream_t s) {
+  constexpr int E = Row16<DT>::kElems;
+  if (H % E != 0) return OMNI_ERR_SHAPE;              // rows must be 16-byte multiples
+  const int nch = (H + kWave * E - 1) / (kWave * E);
+  hipError_t err;
+  if (nch <= 1) err = launch_gather<DT, 1, 16>(x, up, down, gates, ids, y, T, H, k, N, s);
+  else if (nch <= 2) err = launch_gather<DT, 2, 8>(x, up, down, gates, ids, y, T, H, k, N, s);
+  else if (nch <= 4) err = launch_gather<DT, 4, 4>(x, up, down, gates, ids, y, T, H, k, N, s);
+  else if (nch <= 8) err = launch_gather<DT, 8, 2>(x, up, down, gates, ids, y, T, H, k, N, s);
+  else return OMNI_ERR_UNSUPPORTED;
+  return err == hipSuccess ? OMNI_OK : OMNI_ERR_HIP_BASE + (int)err;
+}
+
+}  // namespace omni
+
+extern "C" OMNI_API size_t omni_expert_workspace_bytes(int64_t num_tokens, int32_t hidden_size, int64_t num_experts,
+                                                       int32_t num_experts_per_token, int32_t dtype, int32_t algo) {
+  (void)num_tokens; (void)hidden_size; (void)num_experts; (void)num_experts_per_token; (void)dtype; (void)algo;
+  return 0;   // the gather algorithm keeps everything in registers
+}
+
+extern "C" OMNI_API int32_t omni_expert_fwd(const void* x, const void* up_weight, const void* down_weight,
+                               const void* routing_weights, const int32_t* indices, void* y,
+                               int64_t num_tokens, int32_t hidden_size, int64_t num_experts,
+                               int32_t num_experts_per_token, int32_t dtype, int32_t algo,
+                               void* workspace, void* stream) {
+  using namespace omni;
+  if (num_tokens < 0 || hidden_size <= 0 || num_experts <= 0 || num_experts_per_token < 0) return OMNI_ERR_SHAPE;
+  if (num_tokens > INT32_MAX / 2 || num_experts > UINT32_MAX) return OMNI_ERR_SHAPE;
+  if (num_tokens > 0 && (!x || !up_weight || !down_weight || !y)) return OMNI_ERR_NULL;
+  if (num_tokens > 0 && num_experts_per_token > 0 && (!routing_weights || !indices)) return OMNI_ERR_NULL;
+  hipStream_t s = (hipStream_t)stream;
+  (void)workspace;
+  if (algo != OMNI_EXPERT_ALGO_AUTO && algo != OMNI_EXPERT_ALGO_GATHER) return OMNI_ERR_UNSUPPORTED;
+  switch (dtype) {
+    case OMNI_BF16: return expert_gather_dispatch<kBF16>(x, up_weight, down_weight, routing_weights, indices, y, num_tokens, hidden_size, num_experts_per_token, num_experts, s);
+    case OMNI_F16: return expert_gather_dispatch<kF16>(x, up_weight, down_weight, routing_weights, indices, y, num_tokens, hidden_size, num_experts_per_token, num_experts, s);
+    case OMNI_F32: return expert_gather_dispatch<kF32>(x, up_weight, down_weight, routing_weights, indices, y, num_tokens, hidden_size, num_experts_per_token, num_experts, s);
+    default: return OMNI_ERR_DTYPE;
+  }
+}

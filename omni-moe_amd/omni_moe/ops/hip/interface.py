@@ -1,0 +1,128 @@
+"""Operator API of the OmniMoE forward path on MI355X.
+
+Same call signatures, shapes, dtypes and return arity as the reference's
+``omni_moe/ops/triton/interface.py`` (router :32-51, expert :54-72, mlp :7-29); the
+work is done by hand-written gfx950 kernels behind the C ABI in
+``include/omni_moe_hip.h``.  Forward only.
+"""
+from __future__ import annotations
+
+from typing import NamedTuple, Optional, Tuple
+
+import torch
+
+from . import _lib
+
+
+def _c(t: torch.Tensor) -> torch.Tensor:
+    # the reference makes every tensor argument contiguous (utils.py:47-65)
+    return t if t.is_contiguous() else t.contiguous()
+
+
+def hip_omni_router_func(
+    router_logits_x: torch.Tensor,
+    router_logits_y: torch.Tensor,
+    num_expert_sqrt: int,
+    num_experts_per_token: int,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Cartesian-product top-k: (scores [T,k] in the input dtype, indices [T,k] int32).
+
+    Mirrors ``triton_omni_router_func`` (reference interface.py:32-51) and the input
+    contract of ``assert_omni_router_fwd_inputs`` (utils.py:81-104).
+    """
+    assert router_logits_x.dim() == 2, "router_logits_x must be a 2D tensor of shape (num_tokens, num_expert_sqrt)"
+    assert router_logits_y.dim() == 2, "router_logits_y must be a 2D tensor of shape (num_tokens, num_expert_sqrt)"
+    assert router_logits_x.size(0) == router_logits_y.size(0), (
+        "router_logits_x and router_logits_y must have the same first dimension")
+    r, k = int(num_expert_sqrt), int(num_experts_per_token)
+    assert 0 <= k <= r * r, f"num_experts_per_token should be in [0, {r * r}], but got {k}"
+    assert k <= 128, "num_experts_per_token should be less than or equal to 128"
+    assert k % 2 == 0, "num_experts_per_token should be a multiple of 2"
+    if router_logits_x.size(1) != r or router_logits_y.size(1) != r:
+        raise ValueError("router logits must have num_expert_sqrt columns")
+    if router_logits_x.dtype != router_logits_y.dtype or router_logits_x.dtype not in _lib.DTYPE_CODE:
+        raise TypeError("router logits must share a dtype in {bfloat16, float16, float32}")
+    dev = _lib.require_gpu(router_logits_x, router_logits_y)
+    lx, ly = _c(router_logits_x), _c(router_logits_y)
+    T = lx.size(0)
+    scores = torch.empty((T, k), device=dev, dtype=lx.dtype)
+    indices = torch.empty((T, k), device=dev, dtype=torch.int32)
+    with torch.cuda.device(dev):
+        code = _lib.load().omni_router_select(
+            _lib.ptr(lx), _lib.ptr(ly), _lib.ptr(scores), _lib.ptr(indices), T, r, k,
+            _lib.DTYPE_CODE[lx.dtype], _lib.stream_ptr())
+    _lib.check(code, "omni_router_select")
+    return scores, indices
+
+
+class Schedule(NamedTuple):
+    """Expert-centric layout of the (token, expert) pairs (dense form of the reference's
+    ``SchedulingInfo`` tail fields, omni_scheduler.py:5-43)."""
+    offsets: torch.Tensor            # [N+1] int32
+    sorted_pair_ids: torch.Tensor    # [T*k] int32
+    sorted_token_ids: torch.Tensor   # [T*k] int32
+
+
+def hip_omni_schedule_func(indices: torch.Tensor, num_experts: int) -> Schedule:
+    """Counting sort of the pairs by expert id; no device-to-host traffic.
+
+    Stands in for ``get_scheduling_info(G, Indices, num_experts, group_size)``
+    (reference omni_scheduler.py:48-101, tail part).
+    """
+    if indices.dim() != 2 or indices.dtype != torch.int32:
+        raise TypeError("indices must be a 2D int32 tensor (num_tokens, num_experts_per_token)")
+    dev = _lib.require_gpu(indices)
+    idx = _c(indices)
+    T, k = idx.shape
+    N = int(num_experts)
+    lib = _lib.load()
+    offsets = torch.empty(N + 1, device=dev, dtype=torch.int32)
+    pair_ids = torch.empty(T * k, device=dev, dtype=torch.int32)
+    token_ids = torch.empty(T * k, device=dev, dtype=torch.int32)
+    ws = torch.empty(max(lib.omni_schedule_workspace_bytes(T, k, N), 1), device=dev, dtype=torch.uint8)
+    with torch.cuda.device(dev):
+        code = lib.omni_schedule(_lib.ptr(idx), _lib.ptr(offsets), _lib.ptr(pair_ids), _lib.ptr(token_ids),
+                                 T, k, N, _lib.ptr(ws), _lib.stream_ptr())
+    _lib.check(code, "omni_schedule")
+    return Schedule(offsets, pair_ids, token_ids)
+
+
+_ALGOS = {"auto": _lib.ALGO_AUTO, "gather": _lib.ALGO_GATHER, "segment": _lib.ALGO_SEGMENT}
+
+
+def hip_omni_expert_func(
+    x: torch.Tensor,
+    up_weight: torch.Tensor,
+    down_weight: torch.Tensor,
+    routing_weights: torch.Tensor,
+    indices: torch.Tensor,
+    algo: str = "auto",
+) -> torch.Tensor:
+    """y[t] = sum_j silu(<x[t], up[idx_tj]>) * g_tj * down[idx_tj];  y has x's shape and dtype.
+
+    Mirrors ``triton_omni_expert_func`` (reference interface.py:54-72).
+    """
+    if x.dim() != 2 or up_weight.dim() != 2 or down_weight.dim() != 2:
+        raise ValueError("x, up_weight and down_weight must be 2D")
+    if routing_weights.shape != indices.shape or routing_weights.dim() != 2 or routing_weights.size(0) != x.size(0):
+        raise ValueError("routing_weights and indices must both be (num_tokens, num_experts_per_token)")
+    if up_weight.shape != down_weight.shape or up_weight.size(1) != x.size(1):
+        raise ValueError("up_weight and down_weight must both be (num_experts, hidden_size)")
+    if x.dtype not in _lib.DTYPE_CODE or any(t.dtype != x.dtype for t in (up_weight, down_weight, routing_weights)):
+        raise TypeError("x, up_weight, down_weight, routing_weights must share a dtype in {bfloat16, float16, float32}")
+    if indices.dtype != torch.int32:
+        indices = indices.to(torch.int32)
+    dev = _lib.require_gpu(x, up_weight, down_weight, routing_weights, indices)
+    x, up_weight, down_weight, routing_weights, indices = map(_c, (x, up_weight, down_weight, routing_weights, indices))
+    T, H = x.shape
+    N, k = up_weight.size(0), indices.size(1)
+    lib = _lib.load()
+    dt, al = _lib.DTYPE_CODE[x.dtype], _ALGOS[algo]
+    y = torch.empty_like(x)
+    nbytes = lib.omni_expert_workspace_bytes(T, H, N, k, dt, al)
+    ws = torch.empty(nbytes, device=dev, dtype=torch.uint8) if nbytes else None
+    with torch.cuda.device(dev):
+        code = lib.omni_expert_fwd(_lib.ptr(x), _lib.ptr(up_weight), _lib.ptr(down_weight), _lib.ptr(routing_weights),
+                                   _lib.ptr(indices), _lib.ptr(y), T, H, N, k, dt, al, _lib.ptr(ws), _lib.stream_ptr())
+    _lib.check(code, "omni_expert_fwd")
+    return y

@@ -1,0 +1,187 @@
+"""GPU parity of the HIP operators against the CPU oracle (same seeded inputs).
+
+Every call goes through the C ABI (ctypes -> libomni_moe_hip.so).  Bars:
+index / integer results bit-exact; scores bit-exact (they are sums of two inputs
+rounded once); floating outputs within rtol=atol=2e-2 for 16-bit storage and
+1e-4 / 1e-5 for fp32 storage.
+"""
+import pytest
+import torch
+
+from oracle import omni_oracle as oracle
+
+pytestmark = pytest.mark.gpu
+
+
+def _ops():
+    from omni_moe.ops import hip
+    return hip
+
+
+# ---------------------------------------------------------------- router select
+ROUTER_CASES = [
+    # (T, r, k, dtype, kind)  -- first six are the reference benchmark grid (tests/test_router.py:103-110)
+    (1024, 64, 16, torch.bfloat16, "randn"),
+    (1024, 64, 32, torch.bfloat16, "randn"),
+    (1024, 128, 16, torch.bfloat16, "randn"),
+    (1024, 128, 32, torch.bfloat16, "randn"),
+    (1024, 256, 16, torch.bfloat16, "randn"),
+    (1024, 256, 32, torch.bfloat16, "randn"),
+    (4096, 64, 16, torch.bfloat16, "logprob"),     # BASELINE config 2 shape
+    (2048, 512, 32, torch.bfloat16, "logprob"),    # BASELINE config 5 shape (token subset)
+    (512, 32, 8, torch.float32, "logprob"),        # BASELINE config 1 shape
+    (333, 64, 16, torch.float16, "randn"),
+    (257, 100, 10, torch.bfloat16, "randn"),       # r not a multiple of 64
+    (64, 4, 16, torch.bfloat16, "randn"),          # k = r*r: every expert selected, k' = r
+    (64, 8, 32, torch.float32, "randn"),           # k > r
+    (100, 128, 128, torch.bfloat16, "randn"),      # largest k the contract allows
+    (100, 1024, 64, torch.bfloat16, "randn"),      # largest r the kernel covers
+    (512, 64, 16, torch.bfloat16, "ties"),         # heavy ties: scores on a coarse grid
+    (512, 64, 16, torch.float32, "allequal"),      # all scores equal: pure tie-break
+    (1, 64, 2, torch.bfloat16, "randn"),
+]
+
+
+def _router_inputs(T, r, dtype, kind, seed):
+    g = torch.Generator().manual_seed(seed)
+    a, b = torch.randn(T, r, generator=g), torch.randn(T, r, generator=g)
+    if kind == "logprob":
+        a, b = torch.log_softmax(a, -1), torch.log_softmax(b, -1)
+    elif kind == "ties":
+        a, b = (a * 2).round() / 2, (b * 2).round() / 2
+    elif kind == "allequal":
+        a, b = torch.zeros(T, r), torch.zeros(T, r)
+    return a.to(dtype), b.to(dtype)
+
+
+@pytest.mark.parametrize("case", ROUTER_CASES, ids=lambda c: f"T{c[0]}-r{c[1]}-k{c[2]}-{str(c[3]).split('.')[-1]}-{c[4]}")
+def test_router_select_bit_exact(case, device):
+    T, r, k, dtype, kind = case
+    lx, ly = _router_inputs(T, r, dtype, kind, seed=T + r + k)
+    print(f"router_select T={T} r={r} k={k} {dtype} {kind}", flush=True)
+    want_s, want_i = oracle.router_select(lx, ly, r, k)
+    got_s, got_i = _ops().hip_omni_router_func(lx.to(device), ly.to(device), r, k)
+    torch.cuda.synchronize()
+    assert got_s.dtype == dtype and got_i.dtype == torch.int32 and got_s.shape == (T, k)
+    assert torch.equal(got_s.cpu().float(), want_s.float())
+    assert torch.equal(got_i.cpu(), want_i)
+
+
+def test_router_select_contract(device):
+    hip = _ops()
+    lx = torch.zeros(4, 8, device=device)
+    with pytest.raises(AssertionError):
+        hip.hip_omni_router_func(lx, lx, 8, 3)          # odd k
+    with pytest.raises(AssertionError):
+        hip.hip_omni_router_func(lx, lx, 8, 66)         # k > r*r
+    with pytest.raises(AssertionError):
+        hip.hip_omni_router_func(lx, lx[:2], 8, 4)      # token counts differ
+    s, i = hip.hip_omni_router_func(lx, lx, 8, 0)       # k = 0 is legal: empty result
+    assert s.shape == (4, 0) and i.shape == (4, 0)
+    s, i = hip.hip_omni_router_func(lx[:0], lx[:0], 8, 4)
+    assert s.shape == (0, 4)
+    # non-contiguous input is copied, as the reference does
+    wide = torch.randn(16, 128, device=device)
+    s1, i1 = hip.hip_omni_router_func(wide[:, ::2], wide[:, 1::2], 64, 16)
+    s2, i2 = hip.hip_omni_router_func(wide[:, ::2].contiguous(), wide[:, 1::2].contiguous(), 64, 16)
+    assert torch.equal(s1, s2) and torch.equal(i1, i2)
+
+
+# ---------------------------------------------------------------- schedule
+SCHED_CASES = [(512, 8, 1024, "uniform"), (4096, 16, 4096, "uniform"), (16384, 16, 4096, "uniform"),
+               (4096, 32, 262144, "zipf"), (1000, 6, 5000, "zipf"), (3, 2, 7, "uniform"), (2048, 16, 64, "hot")]
+
+
+def _sched_ids(T, k, N, kind, seed):
+    g = torch.Generator().manual_seed(seed)
+    if kind == "uniform":
+        return torch.randint(0, N, (T, k), generator=g, dtype=torch.int32)
+    if kind == "hot":
+        return torch.zeros(T, k, dtype=torch.int32)
+    w = 1.0 / torch.arange(1, N + 1, dtype=torch.float64) ** 1.1
+    return torch.multinomial(w, T * k, replacement=True, generator=g).reshape(T, k).to(torch.int32)
+
+
+@pytest.mark.parametrize("case", SCHED_CASES, ids=lambda c: f"T{c[0]}-k{c[1]}-N{c[2]}-{c[3]}")
+def test_schedule_matches_oracle(case, device):
+    T, k, N, kind = case
+    ids = _sched_ids(T, k, N, kind, seed=T + k)
+    print(f"schedule T={T} k={k} N={N} {kind}", flush=True)
+    want_off, want_pairs, want_tok = oracle.schedule(ids, N)
+    got = _ops().hip_omni_schedule_func(ids.to(device), N)
+    torch.cuda.synchronize()
+    off, pairs, tok = got.offsets.cpu(), got.sorted_pair_ids.cpu(), got.sorted_token_ids.cpu()
+    assert torch.equal(off, want_off)
+    # the pairs are a permutation, grouped by expert; inside a segment the order is free
+    # (as with the reference's torch.sort) -> compare after ordering each segment
+    flat = ids.reshape(-1).long()
+    assert torch.equal(flat[pairs.long()], flat[want_pairs.long()])
+    key = flat[pairs.long()] * (T * k) + pairs.long()
+    canon = pairs[torch.argsort(key)]
+    assert torch.equal(canon, want_pairs)
+    assert torch.equal(tok, (pairs // k).to(torch.int32))
+
+
+# ---------------------------------------------------------------- expert
+EXPERT_CASES = [
+    # (T, H, N, k, dtype, kind)
+    (1024, 1024, 1024, 32, torch.bfloat16, "ref"),      # reference benchmark grid (tests/test_expert.py:181-187)
+    (1024, 1024, 4096, 32, torch.bfloat16, "ref"),
+    (2048, 1024, 4096, 16, torch.bfloat16, "baseline"), # BASELINE config 3 shape (token subset)
+    (512, 256, 1024, 8, torch.float32, "baseline"),     # BASELINE config 1 shape
+    (256, 2048, 8192, 32, torch.bfloat16, "baseline"),  # BASELINE config 5 row length
+    (130, 1024, 512, 6, torch.float16, "ref"),
+    (77, 520, 300, 10, torch.bfloat16, "ref"),          # H not a multiple of 512
+    (64, 4096, 256, 4, torch.bfloat16, "ref"),
+    (5, 64, 16, 2, torch.float32, "ref"),
+]
+
+
+def _expert_inputs(T, H, N, k, dtype, kind, seed):
+    if kind == "baseline":
+        return oracle.make_expert_inputs(seed, T, H, N, k, dtype)
+    # the reference's benchmark distribution (tests/test_expert.py:83-98): negative gates
+    # occur, ids are drawn with replacement so a token can repeat an expert
+    g = torch.Generator().manual_seed(seed)
+    x = (torch.randn(T, H, generator=g) * 0.5).to(dtype)
+    up = (torch.randn(N, H, generator=g) * 0.1).to(dtype)
+    down = (torch.randn(N, H, generator=g) * 0.1).to(dtype)
+    gates = (torch.randn(T, k, generator=g) * 0.1).to(dtype)
+    ids = torch.randint(0, N, (T, k), generator=g, dtype=torch.int32)
+    return x, up, down, gates, ids
+
+
+def _tol(dtype):
+    return dict(rtol=2e-2, atol=2e-2) if dtype != torch.float32 else dict(rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize("case", EXPERT_CASES, ids=lambda c: f"T{c[0]}-H{c[1]}-N{c[2]}-k{c[3]}-{str(c[4]).split('.')[-1]}-{c[5]}")
+def test_expert_matches_oracle(case, device):
+    T, H, N, k, dtype, kind = case
+    x, up, down, gates, ids = _expert_inputs(T, H, N, k, dtype, kind, seed=T + H)
+    print(f"expert T={T} H={H} N={N} k={k} {dtype} {kind}", flush=True)
+    want = oracle.expert_forward(x, up, down, gates, ids)                 # fp32 sums, one rounding
+    got = _ops().hip_omni_expert_func(*(t.to(device) for t in (x, up, down, gates, ids)))
+    torch.cuda.synchronize()
+    assert got.dtype == dtype and got.shape == (T, H)
+    torch.testing.assert_close(got.cpu().float(), want.float(), **_tol(dtype))
+    # tighter, scale-aware check: the two differ only by fp32 summation order + one rounding
+    err = (got.cpu().float() - want.float()).abs().max().item()
+    scale = want.float().abs().max().item()
+    assert err <= (1e-2 if dtype != torch.float32 else 1e-5) * max(scale, 1e-6), (err, scale)
+
+
+def test_expert_edge_cases(device):
+    hip = _ops()
+    x, up, down, gates, ids = (t.to(device) for t in _expert_inputs(16, 256, 32, 4, torch.bfloat16, "ref", 1))
+    assert hip.hip_omni_expert_func(x[:0], up, down, gates[:0], ids[:0]).shape == (0, 256)       # no tokens
+    y0 = hip.hip_omni_expert_func(x, up, down, gates[:, :0], ids[:, :0])                         # k = 0 -> zeros
+    assert torch.count_nonzero(y0).item() == 0
+    y1 = hip.hip_omni_expert_func(x, up, down, gates, ids)
+    y2 = hip.hip_omni_expert_func(x, up, down, gates, ids)
+    assert torch.equal(y1, y2)                                                                   # deterministic
+    perm = torch.tensor([2, 0, 3, 1], device=device)
+    y3 = hip.hip_omni_expert_func(x, up, down, gates[:, perm].contiguous(), ids[:, perm].contiguous())
+    torch.testing.assert_close(y3.float(), y1.float(), rtol=2e-2, atol=1e-3)                     # slot order is free
+    with pytest.raises(ValueError):
+        hip.hip_omni_expert_func(x, up, down[:, :128], gates, ids)
