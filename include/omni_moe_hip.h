@@ -98,6 +98,55 @@ OMNI_API int32_t omni_expert_fwd(const void* x, const void* up_weight, const voi
                         int32_t num_experts_per_token, int32_t dtype, int32_t algo,
                         void* workspace, void* stream);
 
+/* Shared SwiGLU MLP  y = (silu(x Wg^T) * (x Wu^T)) Wd^T  [+ residual].
+ * Replaces triton_omni_mlp_func (interface.py:7-29: three torch.matmul around the SwiGLU
+ * kernel omni_mlp.py:102-177).  Two MFMA GEMMs: gate/up with the SwiGLU product formed in
+ * the epilogue (gate and up are rounded to the storage dtype, the product is fp32, rounded
+ * once, as omni_mlp.py:53-61), then the down projection.
+ *   x [T,H]; gate_weight, up_weight [I,H]; down_weight [H,I]; y [T,H]  (dtype bf16 or f16)
+ *   residual : NULL, or [T,H] added to the rounded down projection and rounded again
+ *              (the layer's final  mlp + experts , omni_moe.py:102)
+ *   workspace: omni_mlp_workspace_bytes() bytes (the [T,I] SwiGLU activations)
+ * H and I must be multiples of 8. */
+OMNI_API size_t omni_mlp_workspace_bytes(int64_t num_tokens, int32_t hidden_size, int32_t intermediate_size, int32_t dtype);
+OMNI_API int32_t omni_mlp_fwd(const void* x, const void* gate_weight, const void* up_weight, const void* down_weight,
+                              const void* residual, void* y, int64_t num_tokens, int32_t hidden_size,
+                              int32_t intermediate_size, int32_t dtype, void* workspace, void* stream);
+
+/* Bias-free linear layer  y[T,out] = x[T,in] weight[out,in]^T  on the matrix cores.
+ * Replaces the nn.Linear router projections (omni_moe/modules/omni_moe.py:47-52,70-71).
+ * in_features a multiple of 8, out_features of 4; dtype bf16 or f16. */
+OMNI_API int32_t omni_linear_fwd(const void* x, const void* weight, void* y, int64_t num_tokens, int32_t in_features,
+                                 int32_t out_features, int32_t dtype, void* stream);
+
+/* Two bias-free linear layers sharing their input, written side by side:
+ * y[T, 2*out] = [x weight_lo^T | x weight_hi^T].  One GEMM for the router's x and y
+ * projections (omni_moe.py:70-71).  out_features_each a multiple of 2. */
+OMNI_API int32_t omni_linear2_fwd(const void* x, const void* weight_lo, const void* weight_hi, void* y,
+                                  int64_t num_tokens, int32_t in_features, int32_t out_features_each,
+                                  int32_t dtype, void* stream);
+
+/* Router of the layer, from hidden states to gates and expert ids:
+ * projection -> BatchNorm1d(affine=False) -> log_softmax -> Cartesian top-k -> exp.
+ * Replaces omni_moe/modules/omni_moe.py:70-86 (two nn.Linear, two nn.BatchNorm1d, two
+ * F.log_softmax, triton_omni_router_func, torch.exp).  Every stage rounds to the storage
+ * dtype where the torch ops do.
+ *   x [T,H]; weight_x, weight_y [r,H]                                     (dtype bf16 or f16)
+ *   running_mean_*, running_var_* [r] of dtype stats_dtype; num_batches_tracked_* int64
+ *     scalars (may be NULL).  training != 0: batch statistics normalise (biased variance)
+ *     and the buffers are UPDATED in place with `momentum` (unbiased variance), as
+ *     nn.BatchNorm1d in train mode; training == 0: the buffers normalise, nothing is written.
+ *   gates [T,k] dtype = exp(score); indices [T,k] int32; scores [T,k] dtype or NULL
+ *   workspace: omni_router_workspace_bytes() bytes */
+OMNI_API size_t omni_router_workspace_bytes(int64_t num_tokens, int32_t num_expert_sqrt, int32_t dtype);
+OMNI_API int32_t omni_router_fwd(const void* x, const void* weight_x, const void* weight_y,
+                                 void* running_mean_x, void* running_var_x, int64_t* num_batches_tracked_x,
+                                 void* running_mean_y, void* running_var_y, int64_t* num_batches_tracked_y,
+                                 int32_t training, float momentum, float eps, void* gates, int32_t* indices,
+                                 void* scores, int64_t num_tokens, int32_t hidden_size, int32_t num_expert_sqrt,
+                                 int32_t num_experts_per_token, int32_t dtype, int32_t stats_dtype,
+                                 void* workspace, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,340 @@
+// MFMA GEMMs of the OmniMoE forward path for gfx950 (C = A * B^T, both operands with K
+// contiguous, fp32 accumulation on the matrix cores):
+//   * router projection   z  = x [Wx;Wy]^T                    (reference omni_moe.py:70-71)
+//   * gate/up projection  h  = silu(x Wg^T) * (x Wu^T)         (interface.py:23-29, omni_mlp.py:53-61)
+//     - the SwiGLU product is formed in the GEMM epilogue, so gate and up never reach HBM
+//   * down projection     y  = h Wd^T (+ expert output)        (interface.py:23-29, omni_moe.py:102)
+//
+// Structure: a block of 4 waves (2 x 2) owns a (2*TM*32) x (2*TN*32) tile; each wave owns
+// TM x TN MFMA tiles of 32x32.  K advances 64 at a time: global 128-bit loads go to
+// registers, then into one of two LDS stages whose rows are padded by 16 bytes so that the
+// 128-bit fragment reads of 16 consecutive rows hit all 64 banks once.  The weight fragment
+// is the MFMA's first operand, so an accumulator lane holds 4 consecutive output columns of
+// one row and stores them as one 8-byte word.
+#include "common.h"
+#include "omni_moe_hip.h"
+
+namespace omni {
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+
+constexpr int kBK = 64;                       // K elements per LDS stage
+constexpr int kRowBytes = kBK * 2 + 16;       // padded LDS row
+constexpr int kGemmThreads = 256;
+
+enum : int { kEpiPlain = 0, kEpiSwiglu = 1, kEpiResidual = 2 };
+
+template <int DT>
+__device__ __forceinline__ f32x16_t mfma32(const u32x4_t a, const u32x4_t b, const f32x16_t c) {
+  if constexpr (DT == kBF16)
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+}
+
+template <int DT>
+__device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+  if constexpr (DT == kBF16) return pack_bf16(lo, hi);
+  else return pack_f16(lo, hi);
+}
+
+struct GemmArgs {
+  const uint16_t* a;      // [M, K]  activations
+  const uint16_t* b0;     // [N, K]  weights (gate weights for SwiGLU)
+  const uint16_t* b1;     // [N, K]  up weights (SwiGLU only)
+  const uint16_t* res;    // [M, N]  added to the result (residual epilogue only)
+  uint16_t* c;            // [M, N]
+  int M, N, K;            // N = output columns
+  int tiles_m, tiles_n;
+  int patch_m, patch_n;   // XCD patch shape (0 = plain order)
+};
+
+// 16-bit storage, TM x TN MFMA tiles per wave.  For the SwiGLU epilogue the first TN/2
+// tiles of a wave are gate columns and the last TN/2 the matching up columns.
+template <int DT, int TM, int TN, int EPI>
+__global__ __launch_bounds__(kGemmThreads, 1) void gemm_nt_kernel(const GemmArgs g) {
+  constexpr int BM = 2 * TM * 32;                 // rows of A per block
+  constexpr int BR = 2 * TN * 32;                 // rows of the weight tile in LDS per block
+  constexpr int BN = (EPI == kEpiSwiglu) ? BR / 2 : BR;   // output columns per block
+  constexpr int TNO = (EPI == kEpiSwiglu) ? TN / 2 : TN;  // output tiles per wave along N
+  constexpr int kStageBytes = (BM + BR) * kRowBytes;
+  extern __shared__ __align__(16) uint8_t lds[];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave & 1, wn = wave >> 1;
+
+  // ---- which tile: blocks go round-robin over the 8 XCDs; give each XCD compact
+  // patches of tiles so that the blocks sharing its L2 share operand panels
+  int tile_m, tile_n;
+  {
+    const int b = blockIdx.x;
+    if (g.patch_m > 0) {
+      const int per_patch = g.patch_m * g.patch_n;
+      const int xcd = b & 7, idx = b >> 3;
+      const int patch = (idx / per_patch) * 8 + xcd, within = idx % per_patch;
+      const int patches_m = g.tiles_m / g.patch_m;
+      tile_m = (patch % patches_m) * g.patch_m + within % g.patch_m;
+      tile_n = (patch / patches_m) * g.patch_n + within / g.patch_m;
+    } else {
+      tile_m = b % g.tiles_m;
+      tile_n = b / g.tiles_m;
+    }
+  }
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+  // ---- global -> register staging: thread owns 16-byte chunk (tid%8) of rows tid/8 + 32*p
+  const int ld_chunk = tid & 7, ld_row = tid >> 3;
+  constexpr int PA = BM / 32, PB = BR / 32;
+  const uint16_t* a_ptr[PA];
+  const uint16_t* b_ptr[PB];
+#pragma unroll
+  for (int p = 0; p < PA; ++p) {
+    int row = m0 + p * 32 + ld_row;
+    row = row < g.M ? row : g.M - 1;                     // clamp: tail rows are never stored
+    a_ptr[p] = g.a + (int64_t)row * g.K + ld_chunk * 8;
+  }
+#pragma unroll
+  for (int p = 0; p < PB; ++p) {
+    // LDS weight row p*32+ld_row belongs to wave column p/TN, tile p%TN
+    const int pw = p / TN, pj = p % TN;
+    const uint16_t* base = g.b0;
+    int col;
+    if constexpr (EPI == kEpiSwiglu) {
+      base = (pj < TNO) ? g.b0 : g.b1;
+      col = n0 + pw * (TNO * 32) + (pj % TNO) * 32 + ld_row;
+    } else {
+      col = n0 + p * 32 + ld_row;
+    }
+    col = col < g.N ? col : g.N - 1;
+    if constexpr (EPI == kEpiPlain) {
+      // optional second weight matrix supplies the upper half of the output columns
+      if (g.b1 && col >= g.N / 2) { base = g.b1; col -= g.N / 2; }
+    }
+    b_ptr[p] = base + (int64_t)col * g.K + ld_chunk * 8;
+  }
+  const int lds_wr = ld_row * kRowBytes + ld_chunk * 16;
+
+  u32x4_t ra[PA], rb[PB];
+  auto load_tile = [&](int k0) {
+    const bool ok = k0 + ld_chunk * 8 < g.K;             // K is a multiple of 8: whole chunks
+#pragma unroll
+    for (int p = 0; p < PA; ++p) ra[p] = ok ? *(const u32x4_t*)(a_ptr[p] + k0) : u32x4_t{0, 0, 0, 0};
+#pragma unroll
+    for (int p = 0; p < PB; ++p) rb[p] = ok ? *(const u32x4_t*)(b_ptr[p] + k0) : u32x4_t{0, 0, 0, 0};
+  };
+  auto store_tile = [&](int stage) {
+    uint8_t* sa = lds + stage * kStageBytes;
+    uint8_t* sb = sa + BM * kRowBytes;
+#pragma unroll
+    for (int p = 0; p < PA; ++p) *(u32x4_t*)(sa + p * 32 * kRowBytes + lds_wr) = ra[p];
+#pragma unroll
+    for (int p = 0; p < PB; ++p) *(u32x4_t*)(sb + p * 32 * kRowBytes + lds_wr) = rb[p];
+  };
+
+  f32x16_t acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int q = 0; q < 16; ++q) acc[i][j][q] = 0.f;
+
+  // fragment read offsets: lane reads row (lane%32), 16-byte chunk (lane/32) of a K=16 slab
+  const int frag_off = (lane & 31) * kRowBytes + (lane >> 5) * 16;
+  const int a_frag = (wm * TM * 32) * kRowBytes + frag_off;
+  const int b_frag = BM * kRowBytes + (wn * TN * 32) * kRowBytes + frag_off;
+
+  const int num_kt = (g.K + kBK - 1) / kBK;
+  load_tile(0);
+  store_tile(0);
+  __syncthreads();
+  for (int kt = 0; kt < num_kt; ++kt) {
+    const uint8_t* st = lds + (kt & 1) * kStageBytes;
+    if (kt + 1 < num_kt) load_tile((kt + 1) * kBK);
+#pragma unroll
+    for (int slab = 0; slab < kBK / 16; ++slab) {
+      u32x4_t af[TM], bf[TN];
+#pragma unroll
+      for (int i = 0; i < TM; ++i) af[i] = *(const u32x4_t*)(st + a_frag + i * 32 * kRowBytes + slab * 32);
+#pragma unroll
+      for (int j = 0; j < TN; ++j) bf[j] = *(const u32x4_t*)(st + b_frag + j * 32 * kRowBytes + slab * 32);
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) acc[i][j] = mfma32<DT>(bf[j], af[i], acc[i][j]);
+    }
+    if (kt + 1 < num_kt) store_tile((kt + 1) & 1);
+    __syncthreads();
+  }
+
+  // ---- epilogue.  acc[i][j][q]: row m = lane%32, column n = (q/4)*8 + (lane/32)*4 + q%4
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    const int m = m0 + wm * TM * 32 + i * 32 + (lane & 31);
+    if (m >= g.M) continue;
+#pragma unroll
+    for (int j = 0; j < TNO; ++j) {
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        const int n = n0 + wn * TNO * 32 + j * 32 + q4 * 8 + (lane >> 5) * 4;
+        if (n >= g.N) continue;                          // N is a multiple of 4
+        float v[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          if constexpr (EPI == kEpiSwiglu) {
+            // the reference materialises gate and up in the storage dtype, then forms
+            // silu(gate)*up in fp32 and rounds once (omni_mlp.py:53-61)
+            const float gt = Elem<DT>::round(acc[i][j][q4 * 4 + q]);
+            const float up = Elem<DT>::round(acc[i][j + TNO][q4 * 4 + q]);
+            v[q] = silu_f32(gt) * up;
+          } else {
+            v[q] = acc[i][j][q4 * 4 + q];
+          }
+        }
+        const int64_t o = (int64_t)m * g.N + n;
+        if constexpr (EPI == kEpiResidual) {
+          // y = round(h Wd^T) + e, rounded again: the reference adds two stored tensors
+          const u32x2_t r = *(const u32x2_t*)(g.res + o);
+          const uint32_t r0 = r[0], r1 = r[1];
+          if constexpr (DT == kBF16) {
+            v[0] = Elem<DT>::round(v[0]) + bf16_lo(r0); v[1] = Elem<DT>::round(v[1]) + bf16_hi(r0);
+            v[2] = Elem<DT>::round(v[2]) + bf16_lo(r1); v[3] = Elem<DT>::round(v[3]) + bf16_hi(r1);
+          } else {
+            v[0] = Elem<DT>::round(v[0]) + f16_bits_to_f32(r0 & 0xffff); v[1] = Elem<DT>::round(v[1]) + f16_bits_to_f32(r0 >> 16);
+            v[2] = Elem<DT>::round(v[2]) + f16_bits_to_f32(r1 & 0xffff); v[3] = Elem<DT>::round(v[3]) + f16_bits_to_f32(r1 >> 16);
+          }
+        }
+        u32x2_t w = {pack2<DT>(v[0], v[1]), pack2<DT>(v[2], v[3])};
+        *(u32x2_t*)(g.c + o) = w;
+      }
+    }
+  }
+}
+
+template <int DT, int TM, int TN, int EPI>
+static hipError_t launch_gemm(GemmArgs g, hipStream_t s) {
+  constexpr int BM = 2 * TM * 32, BR = 2 * TN * 32, BN = (EPI == kEpiSwiglu) ? BR / 2 : BR;
+  constexpr int kLds = 2 * (BM + BR) * kRowBytes;
+  g.tiles_m = (g.M + BM - 1) / BM;
+  g.tiles_n = (g.N + BN - 1) / BN;
+  const int blocks = g.tiles_m * g.tiles_n;
+  // one XCD runs 32 blocks at a time: give it 4 x 8 patches when the tile grid allows
+  g.patch_m = g.patch_n = 0;
+  if (blocks % 256 == 0) {
+    if (g.tiles_m % 4 == 0 && g.tiles_n % 8 == 0) { g.patch_m = 4; g.patch_n = 8; }
+    else if (g.tiles_m % 8 == 0 && g.tiles_n % 4 == 0) { g.patch_m = 8; g.patch_n = 4; }
+  }
+  auto kern = gemm_nt_kernel<DT, TM, TN, EPI>;
+  static bool configured = false;                    // idempotent attribute, set once per instantiation
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
+    if (e != hipSuccess) return e;
+    configured = true;
+  }
+  hipLaunchKernelGGL(kern, dim3(blocks), dim3(kGemmThreads), kLds, s, g);
+  return hipGetLastError();
+}
+
+// Shape rules shared by the entry points: K a multiple of 8 (16-byte chunks), N of 4.
+static int check_gemm(int64_t M, int64_t N, int64_t K) {
+  if (M < 0 || N <= 0 || K <= 0 || M > INT32_MAX / 2 || N > INT32_MAX / 2 || K > INT32_MAX / 2) return OMNI_ERR_SHAPE;
+  if (K % 8 != 0 || N % 4 != 0) return OMNI_ERR_SHAPE;
+  return OMNI_OK;
+}
+
+static int to_code(hipError_t e) { return e == hipSuccess ? OMNI_OK : OMNI_ERR_HIP_BASE + (int)e; }
+
+// C[M,N] = A[M,K] B[N,K]^T (+ res), picking the tile shape from the problem size.
+template <int DT>
+static int gemm_plain(const void* a, const void* b, const void* b_hi, const void* res, void* c, int64_t M, int64_t N, int64_t K, hipStream_t s) {
+  if (int e = check_gemm(M, N, K)) return e;
+  if (M == 0) return OMNI_OK;
+  GemmArgs g{(const uint16_t*)a, (const uint16_t*)b, (const uint16_t*)b_hi, (const uint16_t*)res, (uint16_t*)c, (int)M, (int)N, (int)K, 0, 0, 0, 0};
+  const int64_t big = ((M + 255) / 256) * ((N + 255) / 256), mid = ((M + 127) / 128) * ((N + 127) / 128);
+  hipError_t err;
+  if (res) {
+    if (big >= 200) err = launch_gemm<DT, 4, 4, kEpiResidual>(g, s);
+    else if (mid >= 200) err = launch_gemm<DT, 2, 2, kEpiResidual>(g, s);
+    else err = launch_gemm<DT, 1, 1, kEpiResidual>(g, s);
+  } else {
+    if (big >= 200) err = launch_gemm<DT, 4, 4, kEpiPlain>(g, s);
+    else if (mid >= 200) err = launch_gemm<DT, 2, 2, kEpiPlain>(g, s);
+    else err = launch_gemm<DT, 1, 1, kEpiPlain>(g, s);
+  }
+  return to_code(err);
+}
+
+template <int DT>
+static int gemm_swiglu(const void* x, const void* wg, const void* wu, void* h, int64_t M, int64_t I, int64_t K, hipStream_t s) {
+  if (int e = check_gemm(M, I, K)) return e;
+  if (M == 0) return OMNI_OK;
+  GemmArgs g{(const uint16_t*)x, (const uint16_t*)wg, (const uint16_t*)wu, nullptr, (uint16_t*)h, (int)M, (int)I, (int)K, 0, 0, 0, 0};
+  const int64_t big = ((M + 255) / 256) * ((I + 127) / 128);
+  hipError_t err;
+  if (big >= 200) err = launch_gemm<DT, 4, 4, kEpiSwiglu>(g, s);
+  else err = launch_gemm<DT, 2, 2, kEpiSwiglu>(g, s);
+  return to_code(err);
+}
+
+}  // namespace omni
+
+extern "C" OMNI_API size_t omni_mlp_workspace_bytes(int64_t num_tokens, int32_t hidden_size, int32_t intermediate_size, int32_t dtype) {
+  (void)hidden_size;
+  if (num_tokens < 0 || intermediate_size < 0) return 0;
+  const size_t es = dtype == OMNI_F32 ? 4 : 2;
+  return (size_t)num_tokens * (size_t)intermediate_size * es;      // h = silu(gate)*up
+}
+
+extern "C" OMNI_API int32_t omni_mlp_fwd(const void* x, const void* gate_weight, const void* up_weight, const void* down_weight,
+                                         const void* residual, void* y, int64_t num_tokens, int32_t hidden_size,
+                                         int32_t intermediate_size, int32_t dtype, void* workspace, void* stream) {
+  using namespace omni;
+  if (num_tokens < 0 || hidden_size <= 0 || intermediate_size <= 0) return OMNI_ERR_SHAPE;
+  if (num_tokens == 0) return OMNI_OK;
+  if (!x || !gate_weight || !up_weight || !down_weight || !y) return OMNI_ERR_NULL;
+  if (!workspace) return OMNI_ERR_WORKSPACE;
+  hipStream_t s = (hipStream_t)stream;
+  int e;
+  switch (dtype) {
+    case OMNI_BF16:
+      if ((e = gemm_swiglu<kBF16>(x, gate_weight, up_weight, workspace, num_tokens, intermediate_size, hidden_size, s))) return e;
+      return gemm_plain<kBF16>(workspace, down_weight, nullptr, residual, y, num_tokens, hidden_size, intermediate_size, s);
+    case OMNI_F16:
+      if ((e = gemm_swiglu<kF16>(x, gate_weight, up_weight, workspace, num_tokens, intermediate_size, hidden_size, s))) return e;
+      return gemm_plain<kF16>(workspace, down_weight, nullptr, residual, y, num_tokens, hidden_size, intermediate_size, s);
+    case OMNI_F32: return OMNI_ERR_UNSUPPORTED;
+    default: return OMNI_ERR_DTYPE;
+  }
+}
+
+extern "C" OMNI_API int32_t omni_linear_fwd(const void* x, const void* weight, void* y, int64_t num_tokens, int32_t in_features,
+                                            int32_t out_features, int32_t dtype, void* stream) {
+  using namespace omni;
+  if (num_tokens == 0) return OMNI_OK;
+  if (!x || !weight || !y) return OMNI_ERR_NULL;
+  hipStream_t s = (hipStream_t)stream;
+  switch (dtype) {
+    case OMNI_BF16: return gemm_plain<kBF16>(x, weight, nullptr, nullptr, y, num_tokens, out_features, in_features, s);
+    case OMNI_F16: return gemm_plain<kF16>(x, weight, nullptr, nullptr, y, num_tokens, out_features, in_features, s);
+    case OMNI_F32: return OMNI_ERR_UNSUPPORTED;
+    default: return OMNI_ERR_DTYPE;
+  }
+}
+
+extern "C" OMNI_API int32_t omni_linear2_fwd(const void* x, const void* weight_lo, const void* weight_hi, void* y,
+                                             int64_t num_tokens, int32_t in_features, int32_t out_features_each,
+                                             int32_t dtype, void* stream) {
+  using namespace omni;
+  if (num_tokens == 0) return OMNI_OK;
+  if (!x || !weight_lo || !weight_hi || !y) return OMNI_ERR_NULL;
+  hipStream_t s = (hipStream_t)stream;
+  const int64_t n = 2 * (int64_t)out_features_each;
+  switch (dtype) {
+    case OMNI_BF16: return gemm_plain<kBF16>(x, weight_lo, weight_hi, nullptr, y, num_tokens, n, in_features, s);
+    case OMNI_F16: return gemm_plain<kF16>(x, weight_lo, weight_hi, nullptr, y, num_tokens, n, in_features, s);
+    case OMNI_F32: return OMNI_ERR_UNSUPPORTED;
+    default: return OMNI_ERR_DTYPE;
+  }
+}

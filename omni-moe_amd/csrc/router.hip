@@ -118,14 +118,47 @@ __device__ __forceinline__ void store_score(void* p, int64_t i, float v, int dt)
 constexpr int kRouterWaves = 4;
 constexpr float kNegInf = -__builtin_huge_valf();
 
+struct SelectArgs {
+  const void* lx;        // x-half scores of token t at lx[t*row_stride + key]
+  const void* ly;
+  int64_t row_stride;
+  const float* stats;    // NULL, or [4][r] fp32: mean_x, rstd_x, mean_y, rstd_y -> the inputs are raw
+                         // projections; normalise and log-softmax them before selecting
+  void* scores;          // [T,k] storage dtype, may be NULL
+  void* gates;           // [T,k] storage dtype = exp(score), may be NULL
+  int32_t* indices;      // [T,k]
+  int num_tokens, r, k, kp, dt;
+};
+
+// BatchNorm (affine-free) then log-softmax of one half, in place: v holds the raw projection
+// of key a*64+lane (NaN-free -inf padding past r).  Each stage rounds to the storage dtype
+// where the reference's torch ops do (BN output, log-softmax output; omni_moe.py:70-78).
+template <int R>
+__device__ __forceinline__ void normalise_half(float (&v)[R], const float* mean, const float* rstd, int r, int lane, int dt) {
+  float m = kNegInf;
+#pragma unroll
+  for (int a = 0; a < R; ++a) {
+    const int key = a * kWave + lane;
+    if (key < r) v[a] = round_score((v[a] - mean[key]) * rstd[key], dt);
+    m = fmaxf(m, v[a]);
+  }
+  m = wave_max(m);
+  float e = 0.f;
+#pragma unroll
+  for (int a = 0; a < R; ++a) e += (a * kWave + lane < r) ? expf(v[a] - m) : 0.f;
+  const float lse = logf(wave_sum(e));
+#pragma unroll
+  for (int a = 0; a < R; ++a)
+    if (a * kWave + lane < r) v[a] = round_score(v[a] - m - lse, dt);
+}
+
 // R = half keys per lane (r <= 64*R); C = candidate cells per lane.
 template <int R, int C>
-__global__ __launch_bounds__(kRouterWaves* kWave) void router_select_kernel(
-    const void* __restrict__ lx, const void* __restrict__ ly, void* __restrict__ scores,
-    int32_t* __restrict__ indices, int num_tokens, int r, int k, int kp, int dt) {
+__global__ __launch_bounds__(kRouterWaves* kWave) void router_select_kernel(const SelectArgs g) {
   const int lane = lane_id();
   const int wave = blockIdx.x * kRouterWaves + (threadIdx.x >> 6);
   const int num_waves = gridDim.x * kRouterWaves;
+  const int r = g.r, k = g.k, kp = g.kp, dt = g.dt;
 
   // This lane's candidate cells: cell index ci = c*64+lane enumerates rows a = 0..kp-1
   // with min(kp, k/(a+1)) cells each.  Payload (a<<8)|b orders like position a*kp+b.
@@ -141,16 +174,20 @@ __global__ __launch_bounds__(kRouterWaves* kWave) void router_select_kernel(
     }
   }
 
-  for (int t = wave; t < num_tokens; t += num_waves) {
+  for (int t = wave; t < g.num_tokens; t += num_waves) {
     float sx[R], sy[R];
     int px[R], py[R];
 #pragma unroll
     for (int a = 0; a < R; ++a) {
       const int key = a * kWave + lane;
       const bool ok = key < r;
-      sx[a] = ok ? load_score(lx, int64_t(t) * r + key, dt) : kNegInf;
-      sy[a] = ok ? load_score(ly, int64_t(t) * r + key, dt) : kNegInf;
+      sx[a] = ok ? load_score(g.lx, int64_t(t) * g.row_stride + key, dt) : kNegInf;
+      sy[a] = ok ? load_score(g.ly, int64_t(t) * g.row_stride + key, dt) : kNegInf;
       px[a] = py[a] = key;
+    }
+    if (g.stats) {
+      normalise_half<R>(sx, g.stats, g.stats + r, r, lane, dt);
+      normalise_half<R>(sy, g.stats + 2 * r, g.stats + 3 * r, r, lane, dt);
     }
     bitonic_sort<R>(sx, px, lane);
     bitonic_sort<R>(sy, py, lane);
@@ -175,8 +212,10 @@ __global__ __launch_bounds__(kRouterWaves* kWave) void router_select_kernel(
       const int a = ok ? (cp[c] >> 8) & 255 : 0, b = ok ? (cp[c] & 255) : 0;
       const int ia = sorted_item<R>(px, a), ib = sorted_item<R>(py, b);
       if (ok) {
-        store_score(scores, int64_t(t) * k + j, cs[c], dt);
-        indices[int64_t(t) * k + j] = ia * r + ib;
+        const int64_t o = int64_t(t) * k + j;
+        if (g.scores) store_score(g.scores, o, cs[c], dt);
+        if (g.gates) store_score(g.gates, o, expf(cs[c]), dt);      // gate = P(x key) * P(y key)
+        g.indices[o] = ia * r + ib;
       }
     }
   }
@@ -189,45 +228,117 @@ static int num_cells(int k, int kp) {
 }
 
 template <int R, int C>
-static hipError_t launch_select(const void* lx, const void* ly, void* scores, int32_t* indices, int64_t T,
-                                int r, int k, int kp, int dt, hipStream_t s) {
-  int64_t blocks = (T + kRouterWaves - 1) / kRouterWaves;
+static hipError_t launch_select(const SelectArgs& g, hipStream_t s) {
+  int64_t blocks = ((int64_t)g.num_tokens + kRouterWaves - 1) / kRouterWaves;
   if (blocks > 256 * 16) blocks = 256 * 16;     // waves loop over tokens beyond that
-  hipLaunchKernelGGL((router_select_kernel<R, C>), dim3((unsigned)blocks), dim3(kRouterWaves * kWave), 0, s, lx, ly,
-                     scores, indices, (int)T, r, k, kp, dt);
+  hipLaunchKernelGGL((router_select_kernel<R, C>), dim3((unsigned)blocks), dim3(kRouterWaves * kWave), 0, s, g);
   return hipGetLastError();
 }
 
 template <int R>
-static hipError_t select_by_cells(int cpl, const void* lx, const void* ly, void* scores, int32_t* indices,
-                                  int64_t T, int r, int k, int kp, int dt, hipStream_t s) {
-  if (cpl <= 1) return launch_select<R, 1>(lx, ly, scores, indices, T, r, k, kp, dt, s);
-  if (cpl <= 2) return launch_select<R, 2>(lx, ly, scores, indices, T, r, k, kp, dt, s);
-  if (cpl <= 4) return launch_select<R, 4>(lx, ly, scores, indices, T, r, k, kp, dt, s);
-  if (cpl <= 8) return launch_select<R, 8>(lx, ly, scores, indices, T, r, k, kp, dt, s);
-  return launch_select<R, 16>(lx, ly, scores, indices, T, r, k, kp, dt, s);
+static hipError_t select_by_cells(int cpl, const SelectArgs& g, hipStream_t s) {
+  if (cpl <= 1) return launch_select<R, 1>(g, s);
+  if (cpl <= 2) return launch_select<R, 2>(g, s);
+  if (cpl <= 4) return launch_select<R, 4>(g, s);
+  if (cpl <= 8) return launch_select<R, 8>(g, s);
+  return launch_select<R, 16>(g, s);
 }
 
-static int select_dispatch(const void* lx, const void* ly, void* scores, int32_t* indices, int64_t T, int r,
-                           int k, int dt, hipStream_t s) {
-  const int kp = r < k ? r : k;
-  const int cpl = (num_cells(k, kp) + kWave - 1) / kWave;   // <= 11 for k <= 128
-  const int rpl = (r + kWave - 1) / kWave;
+static int select_dispatch(SelectArgs g, hipStream_t s) {
+  g.kp = g.r < g.k ? g.r : g.k;
+  const int cpl = (num_cells(g.k, g.kp) + kWave - 1) / kWave;   // <= 11 for k <= 128
+  const int rpl = (g.r + kWave - 1) / kWave;
   hipError_t err;
-  if (rpl <= 1) err = select_by_cells<1>(cpl, lx, ly, scores, indices, T, r, k, kp, dt, s);
-  else if (rpl <= 2) err = select_by_cells<2>(cpl, lx, ly, scores, indices, T, r, k, kp, dt, s);
-  else if (rpl <= 4) err = select_by_cells<4>(cpl, lx, ly, scores, indices, T, r, k, kp, dt, s);
-  else if (rpl <= 8) err = select_by_cells<8>(cpl, lx, ly, scores, indices, T, r, k, kp, dt, s);
-  else if (rpl <= 16) err = select_by_cells<16>(cpl, lx, ly, scores, indices, T, r, k, kp, dt, s);
+  if (rpl <= 1) err = select_by_cells<1>(cpl, g, s);
+  else if (rpl <= 2) err = select_by_cells<2>(cpl, g, s);
+  else if (rpl <= 4) err = select_by_cells<4>(cpl, g, s);
+  else if (rpl <= 8) err = select_by_cells<8>(cpl, g, s);
+  else if (rpl <= 16) err = select_by_cells<16>(cpl, g, s);
   else return OMNI_ERR_UNSUPPORTED;                          // r > 1024
   return err == hipSuccess ? OMNI_OK : OMNI_ERR_HIP_BASE + (int)err;
 }
 
+// ---- BatchNorm1d(affine=False) statistics over the T rows of z [T, C] -------------------
+constexpr int kBnRows = 32;       // rows per partial
+
+// Partial (mean, M2) of every column over a strip of <= 32 rows, two passes over registers.
+__global__ __launch_bounds__(256) void bn_partial_kernel(const void* __restrict__ z, float* __restrict__ part_mean,
+                                                         float* __restrict__ part_m2, int num_rows, int num_cols, int dt) {
+  const int col = blockIdx.x * 256 + threadIdx.x;
+  if (col >= num_cols) return;
+  const int row0 = blockIdx.y * kBnRows;
+  const int n = min(kBnRows, num_rows - row0);
+  float v[kBnRows], sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < kBnRows; ++i) {
+    v[i] = (i < n) ? load_score(z, int64_t(row0 + i) * num_cols + col, dt) : 0.f;
+    sum += v[i];
+  }
+  const float mean = sum / float(n);
+  float m2 = 0.f;
+#pragma unroll
+  for (int i = 0; i < kBnRows; ++i) {
+    const float d = v[i] - mean;
+    m2 += (i < n) ? d * d : 0.f;
+  }
+  part_mean[int64_t(blockIdx.y) * num_cols + col] = mean;
+  part_m2[int64_t(blockIdx.y) * num_cols + col] = m2;
+}
+
+struct BnFinalArgs {
+  const float* part_mean;   // [strips][2r] (training)
+  const float* part_m2;
+  float* stats;             // [4][r]: mean_x, rstd_x, mean_y, rstd_y
+  void* running_mean[2];    // [r] each, dtype stat_dt; read in eval, updated in training
+  void* running_var[2];
+  int64_t* num_batches_tracked[2];   // may be NULL
+  int num_rows, r, strips, training, stat_dt;
+  float momentum, eps;
+};
+
+// One thread per column: merges the strip partials (Chan's update, in double), writes mean
+// and 1/sqrt(var+eps), and in training moves the running buffers (unbiased variance) as
+// nn.BatchNorm1d does.  In eval the running buffers provide mean and variance.
+__global__ __launch_bounds__(256) void bn_finalize_kernel(const BnFinalArgs g) {
+  const int col = blockIdx.x * 256 + threadIdx.x;
+  if (col == 0 && g.training) {
+    if (g.num_batches_tracked[0]) *g.num_batches_tracked[0] += 1;
+    if (g.num_batches_tracked[1]) *g.num_batches_tracked[1] += 1;
+  }
+  if (col >= 2 * g.r) return;
+  const int half = col >= g.r, key = col - half * g.r;
+  float mean, var;
+  if (g.training) {
+    double n = 0., mu = 0., m2 = 0.;
+    for (int s = 0; s < g.strips; ++s) {
+      const double nb = (double)min(kBnRows, g.num_rows - s * kBnRows);
+      const double mb = g.part_mean[int64_t(s) * 2 * g.r + col], qb = g.part_m2[int64_t(s) * 2 * g.r + col];
+      const double d = mb - mu, nn = n + nb;
+      mu += d * nb / nn;
+      m2 += qb + d * d * n * nb / nn;
+      n = nn;
+    }
+    mean = (float)mu;
+    var = (float)(m2 / n);                                   // biased: normalises the batch
+    const float unbiased = (float)(m2 / (n > 1. ? n - 1. : 1.));
+    const float rm = load_score(g.running_mean[half], key, g.stat_dt), rv = load_score(g.running_var[half], key, g.stat_dt);
+    store_score(g.running_mean[half], key, (1.f - g.momentum) * rm + g.momentum * mean, g.stat_dt);
+    store_score(g.running_var[half], key, (1.f - g.momentum) * rv + g.momentum * unbiased, g.stat_dt);
+  } else {
+    mean = load_score(g.running_mean[half], key, g.stat_dt);
+    var = load_score(g.running_var[half], key, g.stat_dt);
+  }
+  g.stats[(2 * half) * g.r + key] = mean;
+  g.stats[(2 * half + 1) * g.r + key] = 1.0f / sqrtf(var + g.eps);
+}
+
+static inline size_t align256(size_t v) { return (v + 255) / 256 * 256; }
+
 }  // namespace omni
 
 extern "C" OMNI_API int32_t omni_router_select(const void* logits_x, const void* logits_y, void* scores, int32_t* indices,
-                                      int64_t num_tokens, int32_t num_expert_sqrt, int32_t num_experts_per_token,
-                                      int32_t dtype, void* stream) {
+                                               int64_t num_tokens, int32_t num_expert_sqrt, int32_t num_experts_per_token,
+                                               int32_t dtype, void* stream) {
   using namespace omni;
   const int r = num_expert_sqrt, k = num_experts_per_token;
   if (num_tokens < 0 || num_tokens > INT32_MAX / 256 || r <= 0) return OMNI_ERR_SHAPE;
@@ -235,5 +346,57 @@ extern "C" OMNI_API int32_t omni_router_select(const void* logits_x, const void*
   if (dtype != OMNI_BF16 && dtype != OMNI_F16 && dtype != OMNI_F32) return OMNI_ERR_DTYPE;
   if (num_tokens == 0 || k == 0) return OMNI_OK;
   if (!logits_x || !logits_y || !scores || !indices) return OMNI_ERR_NULL;
-  return select_dispatch(logits_x, logits_y, scores, indices, num_tokens, r, k, dtype, (hipStream_t)stream);
+  SelectArgs g{logits_x, logits_y, r, nullptr, scores, nullptr, indices, (int)num_tokens, r, k, 0, dtype};
+  return select_dispatch(g, (hipStream_t)stream);
+}
+
+// workspace layout of omni_router_fwd: z [T,2r] | stats [4r] f32 | part_mean | part_m2
+extern "C" OMNI_API size_t omni_router_workspace_bytes(int64_t num_tokens, int32_t num_expert_sqrt, int32_t dtype) {
+  using namespace omni;
+  if (num_tokens < 0 || num_expert_sqrt <= 0) return 0;
+  const size_t es = dtype == OMNI_F32 ? 4 : 2, r = (size_t)num_expert_sqrt;
+  const size_t strips = ((size_t)num_tokens + kBnRows - 1) / kBnRows;
+  return align256((size_t)num_tokens * 2 * r * es) + align256(4 * r * 4) + 2 * align256(strips * 2 * r * 4);
+}
+
+extern "C" OMNI_API int32_t omni_router_fwd(const void* x, const void* weight_x, const void* weight_y,
+                                            void* running_mean_x, void* running_var_x, int64_t* num_batches_tracked_x,
+                                            void* running_mean_y, void* running_var_y, int64_t* num_batches_tracked_y,
+                                            int32_t training, float momentum, float eps, void* gates, int32_t* indices,
+                                            void* scores, int64_t num_tokens, int32_t hidden_size, int32_t num_expert_sqrt,
+                                            int32_t num_experts_per_token, int32_t dtype, int32_t stats_dtype,
+                                            void* workspace, void* stream) {
+  using namespace omni;
+  const int r = num_expert_sqrt, k = num_experts_per_token;
+  if (num_tokens < 0 || num_tokens > INT32_MAX / 256 || r <= 0 || hidden_size <= 0) return OMNI_ERR_SHAPE;
+  if (k < 0 || (int64_t)k > (int64_t)r * r || k > 128 || (k & 1)) return OMNI_ERR_TOPK;
+  if (dtype != OMNI_BF16 && dtype != OMNI_F16) return dtype == OMNI_F32 ? OMNI_ERR_UNSUPPORTED : OMNI_ERR_DTYPE;
+  if (stats_dtype != OMNI_BF16 && stats_dtype != OMNI_F16 && stats_dtype != OMNI_F32) return OMNI_ERR_DTYPE;
+  if (num_tokens == 0) return OMNI_OK;
+  if (!x || !weight_x || !weight_y || !running_mean_x || !running_var_x || !running_mean_y || !running_var_y) return OMNI_ERR_NULL;
+  if (k > 0 && (!gates || !indices)) return OMNI_ERR_NULL;
+  if (!workspace) return OMNI_ERR_WORKSPACE;
+  hipStream_t s = (hipStream_t)stream;
+  const size_t strips = ((size_t)num_tokens + kBnRows - 1) / kBnRows;
+  char* w = (char*)workspace;
+  void* z = w;                       w += align256((size_t)num_tokens * 2 * r * 2);
+  float* stats = (float*)w;          w += align256((size_t)4 * r * 4);
+  float* part_mean = (float*)w;      w += align256(strips * 2 * r * 4);
+  float* part_m2 = (float*)w;
+
+  // z = x [Wx;Wy]^T on the matrix cores
+  if (int e = omni_linear2_fwd(x, weight_x, weight_y, z, num_tokens, hidden_size, r, dtype, stream)) return e;
+  if (training)
+    hipLaunchKernelGGL(bn_partial_kernel, dim3((2 * r + 255) / 256, (unsigned)strips), dim3(256), 0, s, z, part_mean, part_m2,
+                       (int)num_tokens, 2 * r, dtype);
+  BnFinalArgs b{part_mean, part_m2, stats, {running_mean_x, running_mean_y}, {running_var_x, running_var_y},
+                {num_batches_tracked_x, num_batches_tracked_y}, (int)num_tokens, r, (int)strips, training ? 1 : 0, stats_dtype,
+                momentum, eps};
+  hipLaunchKernelGGL(bn_finalize_kernel, dim3((2 * r + 255) / 256), dim3(256), 0, s, b);
+  hipError_t err = hipGetLastError();
+  if (err != hipSuccess) return OMNI_ERR_HIP_BASE + (int)err;
+  if (k == 0) return OMNI_OK;
+  const size_t es = 2;
+  SelectArgs g{z, (const char*)z + (size_t)r * es, 2 * r, stats, scores, gates, indices, (int)num_tokens, r, k, 0, dtype};
+  return select_dispatch(g, s);
 }

@@ -9,7 +9,7 @@ from __future__ import annotations
 
 import ctypes
 import os
-from ctypes import c_char_p, c_int32, c_int64, c_size_t, c_void_p
+from ctypes import c_char_p, c_float, c_int32, c_int64, c_size_t, c_void_p
 
 import torch  # noqa: F401  (must precede loading the library)
 
@@ -30,6 +30,13 @@ SIGNATURES = {
     "omni_schedule_workspace_bytes": (c_size_t, [c_int64, c_int32, c_int64]),
     "omni_schedule": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int32, c_int64, c_void_p, c_void_p]),
     "omni_expert_workspace_bytes": (c_size_t, [c_int64, c_int32, c_int64, c_int32, c_int32, c_int32]),
+    "omni_mlp_workspace_bytes": (c_size_t, [c_int64, c_int32, c_int32, c_int32]),
+    "omni_mlp_fwd": (c_int32, [c_void_p] * 6 + [c_int64, c_int32, c_int32, c_int32, c_void_p, c_void_p]),
+    "omni_linear_fwd": (c_int32, [c_void_p] * 3 + [c_int64, c_int32, c_int32, c_int32, c_void_p]),
+    "omni_linear2_fwd": (c_int32, [c_void_p] * 4 + [c_int64, c_int32, c_int32, c_int32, c_void_p]),
+    "omni_router_workspace_bytes": (c_size_t, [c_int64, c_int32, c_int32]),
+    "omni_router_fwd": (c_int32, [c_void_p] * 9 + [c_int32, c_float, c_float, c_void_p, c_void_p, c_void_p,
+                                  c_int64, c_int32, c_int32, c_int32, c_int32, c_int32, c_void_p, c_void_p]),
     "omni_expert_fwd": (c_int32, [c_void_p] * 6 + [c_int64, c_int32, c_int64, c_int32, c_int32, c_int32, c_void_p, c_void_p]),
 }
 

@@ -126,3 +126,117 @@ def hip_omni_expert_func(
                                    _lib.ptr(indices), _lib.ptr(y), T, H, N, k, dt, al, _lib.ptr(ws), _lib.stream_ptr())
     _lib.check(code, "omni_expert_fwd")
     return y
+
+
+def hip_omni_mlp_func(
+    x: torch.Tensor,
+    gate_weight: torch.Tensor,
+    up_weight: torch.Tensor,
+    down_weight: torch.Tensor,
+    residual: Optional[torch.Tensor] = None,
+) -> torch.Tensor:
+    """(silu(x gate^T) * (x up^T)) down^T, optionally + residual;  y has x's shape and dtype.
+
+    Mirrors ``triton_omni_mlp_func`` (reference interface.py:7-29).  ``residual`` has no
+    counterpart there: the layer uses it to fold its final ``mlp + experts`` add
+    (omni_moe.py:102) into the down projection's epilogue.
+    """
+    if x.dim() != 2 or gate_weight.dim() != 2 or up_weight.dim() != 2 or down_weight.dim() != 2:
+        raise ValueError("x and the three weights must be 2D")
+    T, H = x.shape
+    I = gate_weight.size(0)
+    if gate_weight.shape != (I, H) or up_weight.shape != (I, H) or down_weight.shape != (H, I):
+        raise ValueError("expected gate/up weights (intermediate, hidden) and down weight (hidden, intermediate)")
+    if x.dtype not in (torch.bfloat16, torch.float16) or any(t.dtype != x.dtype for t in (gate_weight, up_weight, down_weight)):
+        raise TypeError("x and the weights must share a dtype in {bfloat16, float16}")
+    tensors = [x, gate_weight, up_weight, down_weight]
+    if residual is not None:
+        if residual.shape != x.shape or residual.dtype != x.dtype:
+            raise ValueError("residual must match x in shape and dtype")
+        tensors.append(residual)
+    dev = _lib.require_gpu(*tensors)
+    x, gate_weight, up_weight, down_weight = map(_c, (x, gate_weight, up_weight, down_weight))
+    residual = _c(residual) if residual is not None else None
+    lib = _lib.load()
+    dt = _lib.DTYPE_CODE[x.dtype]
+    y = torch.empty_like(x)
+    ws = torch.empty(max(lib.omni_mlp_workspace_bytes(T, H, I, dt), 1), device=dev, dtype=torch.uint8)
+    with torch.cuda.device(dev):
+        code = lib.omni_mlp_fwd(_lib.ptr(x), _lib.ptr(gate_weight), _lib.ptr(up_weight), _lib.ptr(down_weight),
+                                _lib.ptr(residual), _lib.ptr(y), T, H, I, dt, _lib.ptr(ws), _lib.stream_ptr())
+    _lib.check(code, "omni_mlp_fwd")
+    return y
+
+
+def hip_linear_func(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+    """x @ weight.T for a bias-free ``nn.Linear`` (the router projections, reference omni_moe.py:70-71)."""
+    if x.dim() != 2 or weight.dim() != 2 or weight.size(1) != x.size(1):
+        raise ValueError("expected x (tokens, in) and weight (out, in)")
+    if x.dtype not in (torch.bfloat16, torch.float16) or weight.dtype != x.dtype:
+        raise TypeError("x and weight must share a dtype in {bfloat16, float16}")
+    dev = _lib.require_gpu(x, weight)
+    x, weight = _c(x), _c(weight)
+    y = torch.empty((x.size(0), weight.size(0)), device=dev, dtype=x.dtype)
+    with torch.cuda.device(dev):
+        code = _lib.load().omni_linear_fwd(_lib.ptr(x), _lib.ptr(weight), _lib.ptr(y), x.size(0), x.size(1), weight.size(0),
+                                           _lib.DTYPE_CODE[x.dtype], _lib.stream_ptr())
+    _lib.check(code, "omni_linear_fwd")
+    return y
+
+
+def hip_omni_router_fwd_func(
+    x: torch.Tensor,
+    weight_x: torch.Tensor,
+    weight_y: torch.Tensor,
+    running_mean_x: torch.Tensor,
+    running_var_x: torch.Tensor,
+    num_batches_tracked_x: Optional[torch.Tensor],
+    running_mean_y: torch.Tensor,
+    running_var_y: torch.Tensor,
+    num_batches_tracked_y: Optional[torch.Tensor],
+    num_experts_per_token: int,
+    training: bool,
+    momentum: float = 0.1,
+    eps: float = 1e-5,
+    return_scores: bool = False,
+):
+    """Router of the layer in one call: projection -> BatchNorm1d(affine=False) ->
+    log_softmax -> Cartesian top-k -> exp  (reference omni_moe/modules/omni_moe.py:70-86).
+
+    Returns (gates [T,k] in x's dtype, indices [T,k] int32[, scores]).  In training mode the
+    running buffers are updated in place, as nn.BatchNorm1d does.
+    """
+    if x.dim() != 2 or weight_x.shape != weight_y.shape or weight_x.dim() != 2 or weight_x.size(1) != x.size(1):
+        raise ValueError("expected x (tokens, hidden) and two router weights (num_expert_sqrt, hidden)")
+    if x.dtype not in (torch.bfloat16, torch.float16) or weight_x.dtype != x.dtype or weight_y.dtype != x.dtype:
+        raise TypeError("x and the router weights must share a dtype in {bfloat16, float16}")
+    stats = (running_mean_x, running_var_x, running_mean_y, running_var_y)
+    r, k = weight_x.size(0), int(num_experts_per_token)
+    if any(t.dtype != running_mean_x.dtype or t.shape != (r,) or not t.is_contiguous() for t in stats):
+        raise ValueError("running statistics must be contiguous (num_expert_sqrt,) tensors of one dtype")
+    if running_mean_x.dtype not in _lib.DTYPE_CODE:
+        raise TypeError("running statistics must be bfloat16, float16 or float32")
+    assert 0 <= k <= r * r, f"num_experts_per_token should be in [0, {r * r}], but got {k}"
+    assert k <= 128, "num_experts_per_token should be less than or equal to 128"
+    assert k % 2 == 0, "num_experts_per_token should be a multiple of 2"
+    for nbt in (num_batches_tracked_x, num_batches_tracked_y):
+        if nbt is not None and (nbt.dtype != torch.int64 or nbt.numel() != 1):
+            raise TypeError("num_batches_tracked must be an int64 scalar tensor")
+    dev = _lib.require_gpu(x, weight_x, weight_y, *stats)
+    x, weight_x, weight_y = map(_c, (x, weight_x, weight_y))
+    T, H = x.shape
+    lib = _lib.load()
+    dt = _lib.DTYPE_CODE[x.dtype]
+    gates = torch.empty((T, k), device=dev, dtype=x.dtype)
+    indices = torch.empty((T, k), device=dev, dtype=torch.int32)
+    scores = torch.empty((T, k), device=dev, dtype=x.dtype) if return_scores else None
+    ws = torch.empty(max(lib.omni_router_workspace_bytes(T, r, dt), 1), device=dev, dtype=torch.uint8)
+    with torch.cuda.device(dev):
+        code = lib.omni_router_fwd(
+            _lib.ptr(x), _lib.ptr(weight_x), _lib.ptr(weight_y),
+            _lib.ptr(running_mean_x), _lib.ptr(running_var_x), _lib.ptr(num_batches_tracked_x),
+            _lib.ptr(running_mean_y), _lib.ptr(running_var_y), _lib.ptr(num_batches_tracked_y),
+            1 if training else 0, float(momentum), float(eps), _lib.ptr(gates), _lib.ptr(indices), _lib.ptr(scores),
+            T, H, r, k, dt, _lib.DTYPE_CODE[running_mean_x.dtype], _lib.ptr(ws), _lib.stream_ptr())
+    _lib.check(code, "omni_router_fwd")
+    return (gates, indices, scores) if return_scores else (gates, indices)
