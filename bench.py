@@ -2,9 +2,17 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
-Prints ONE JSON line.  A step = one pass of the path over one batch of synthetic,
-HBM-resident input.  Timing uses HIP events recorded on the stream the kernels run on
-(torch's current stream; the library enqueues there).
+Prints ONE JSON line.  A step = one forward of the OmniMoE layer over one batch of synthetic,
+HBM-resident input: BASELINE config 4, the README shape (1 x 4096 tokens, hidden 1024,
+intermediate 4096, 4096 experts = 64 x 64 keys, top-16, bf16, train-mode BatchNorm).
+All timing uses HIP events recorded on the stream the kernels run on (torch's current stream;
+the library enqueues there).
+
+  value      whole-layer tokens/s over the K timed steps
+  roofline   the kernel that takes the largest share of a step (gate/up MFMA GEMM), timed per
+             launch with events around its C-ABI call
+  kernels    the same per-launch figures for every stage of the step, plus the fused expert
+             kernel on BASELINE config 3 (16384 tokens), the shape its bandwidth target is quoted on
 """
 import argparse
 import json
@@ -17,91 +25,159 @@ for p in (os.path.join(ROOT, "omni-moe_amd"), ROOT):
     if p not in sys.path:
         sys.path.insert(0, p)
 
-HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 
 
 def expert_alg_bytes(T, H, k, s=2):
-    # per token: x row + k up rows + k down rows + y row, plus k ids (4 B) and k gates (s B)
+    """Gather model: per token the x row, k up rows, k down rows, the y row, k ids and k gates."""
     return T * ((2 * k + 2) * H * s + k * (4 + s))
+
+
+def _events(torch, n):
+    return [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
+
+
+def time_call(torch, fn, reps, warmup=3):
+    """Mean per-launch milliseconds of fn, HIP events around each call."""
+    for _ in range(warmup):
+        fn()
+    ev = _events(torch, reps)
+    torch.cuda.synchronize()
+    for s, e in ev:
+        s.record()
+        fn()
+        e.record()
+    torch.cuda.synchronize()
+    return sum(s.elapsed_time(e) for s, e in ev) / reps
+
+
+def hbm_entry(name, alg_bytes, ms, note=None):
+    a = alg_bytes / (ms * 1e-3) / 1e9
+    d = {"kernel": name, "bound": "hbm", "achieved": a, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": a / HBM_PEAK_GBS,
+         "traffic": None, "algorithmic_bytes": alg_bytes, "kernel_ms": ms}
+    if note:
+        d["note"] = note
+    return d
+
+
+def mfma_entry(name, flops, ms):
+    a = flops / (ms * 1e-3) / 1e12
+    return {"kernel": name, "bound": "mfma", "achieved": a, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+            "frac": a / MFMA_BF16_PEAK_TFLOPS, "traffic": None, "algorithmic_flops": flops, "kernel_ms": ms}
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel passes (profiling runs)")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU; --gpus must be 1 (no multi-GPU path exists)")
 
     import torch
+    from omni_moe.modules.omni_moe import OmniMoE, OmniMoEConfig
     from omni_moe.ops import hip
     from oracle import omni_oracle as oracle          # checker + cpu_baseline leg only
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 
-    # BASELINE config 3: expert stage incl. the expert-centric sort
-    T, H, N, k, seed = 16384, 1024, 4096, 16, 2
-    x, up, down, gates, ids = oracle.make_expert_inputs(seed, T, H, N, k)
-    dx, dup, ddown, dgates, dids = (t.to(dev) for t in (x, up, down, gates, ids))
-
-    def step():
-        hip.hip_omni_schedule_func(dids, N)
-        return hip.hip_omni_expert_func(dx, dup, ddown, dgates, dids)
+    # ---------------- BASELINE config 4: README-shape full layer
+    T, H, I, N, k, seed = 4096, 1024, 4096, 4096, 16, 3
+    x, w = oracle.make_layer_inputs(seed, T, H, I, N)
+    layer = OmniMoE(OmniMoEConfig(H, I, "silu", N, k))
+    layer.load_state_dict({"gate_proj.weight": w.gate_proj, "up_proj.weight": w.up_proj, "down_proj.weight": w.down_proj,
+                           "router_gate_x.weight": w.router_gate_x, "router_gate_y.weight": w.router_gate_y,
+                           "up_embed.weight": w.up_embed, "down_embed.weight": w.down_embed}, strict=False)
+    layer = layer.to(device=dev, dtype=torch.bfloat16)          # module default: training mode (batch-stat BN)
+    dx = x.to(dev)
 
     for _ in range(a.warmup):
-        y = step()
+        y = layer(dx)
     torch.cuda.synchronize()
-    # spot check against the oracle on a slice (checker, outside the timed region)
-    want = oracle.expert_forward(x[:256], up, down, gates[:256], ids[:256])
-    torch.testing.assert_close(y[:256].cpu().float(), want.float(), rtol=2e-2, atol=2e-2)
 
-    # per-kernel duration of the expert kernel alone (events around each launch)
-    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(a.steps)]
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
     s_all, e_all = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
     s_all.record()
-    for s, e in evs:
-        hip.hip_omni_schedule_func(dids, N)
-        s.record()
-        hip.hip_omni_expert_func(dx, dup, ddown, dgates, dids)
-        e.record()
+    for _ in range(a.steps):
+        y = layer(dx)
     e_all.record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
-    total_ms = s_all.elapsed_time(e_all)
-    ms_per_step = total_ms / a.steps
-    kern_ms = sum(s.elapsed_time(e) for s, e in evs) / a.steps
+    ms_per_step = s_all.elapsed_time(e_all) / a.steps
 
-    alg = expert_alg_bytes(T, H, k)
-    achieved = alg / (kern_ms * 1e-3) / 1e9
     out = {
-        "metric": "OmniMoE expert-stage fwd tokens/sec @h1024,N4096,k16 (1 GPU)",
+        "metric": "OmniMoE fwd tokens/sec @h1024,N4096,k16 (1 GPU); expert kernel HBM GB/s %peak",
         "value": T / (ms_per_step * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": "BASELINE config 3: schedule + fused expert, T=16384 H=1024 N=4096 k=16 bf16 seed 2"},
-        "roofline": {"bound": "hbm", "kernel": "expert_gather_kernel", "achieved": achieved, "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
-                     "algorithmic_bytes": alg, "kernel_ms": kern_ms},
-        "wall_s": wall,
+        "config": {"workload": "BASELINE config 4: full OmniMoE layer forward, 1x4096 tokens, hidden 1024, intermediate 4096, "
+                               "4096 experts (64x64), top-16, silu, train-mode BatchNorm, seed 3"},
+        "wall_s_timed_region": wall,
     }
+
+    # correctness spot check against the oracle (outside the timed region): eval mode on both
+    # sides so that the repeated train-mode steps above do not matter
+    layer.eval()
+    sub = 256
+    y_sub = layer(dx[:, :sub]).float().cpu()
+    bx, by = oracle.BNState.fresh(layer.num_expert_sqrt), oracle.BNState.fresh(layer.num_expert_sqrt)
+    bx.running_mean, bx.running_var = layer.router_norm_x.running_mean.float().cpu(), layer.router_norm_x.running_var.float().cpu()
+    by.running_mean, by.running_var = layer.router_norm_y.running_mean.float().cpu(), layer.router_norm_y.running_var.float().cpu()
+    want, _, _ = oracle.moe_forward(x[:, :sub], w, bx, by, k, training=False)
+    torch.testing.assert_close(y_sub, want.float(), rtol=2e-2, atol=2e-2)
+    layer.train()
+
+    if not a.no_kernels:
+        reps = max(10, min(a.steps, 50))
+        xf = dx.view(-1, H)
+        gates, ids = layer.route(xf)
+        e_out = hip.hip_omni_expert_func(xf, layer.up_embed.weight, layer.down_embed.weight, gates, ids)
+        h = hip.hip_swiglu_linear_func(xf, layer.gate_proj.weight, layer.up_proj.weight)
+        ms_router = time_call(torch, lambda: layer.route(xf), reps)
+        ms_expert = time_call(torch, lambda: hip.hip_omni_expert_func(xf, layer.up_embed.weight, layer.down_embed.weight, gates, ids), reps)
+        ms_gateup = time_call(torch, lambda: hip.hip_swiglu_linear_func(xf, layer.gate_proj.weight, layer.up_proj.weight), reps)
+        ms_down = time_call(torch, lambda: hip.hip_linear_func(h, layer.down_proj.weight, e_out), reps)
+        r = layer.num_expert_sqrt
+        kernels = [
+            mfma_entry("gemm_nt_kernel<swiglu> (gate/up projection + SwiGLU), c4", 4 * T * H * I, ms_gateup),
+            mfma_entry("gemm_nt_kernel<residual> (down projection + experts add), c4", 2 * T * H * I, ms_down),
+            hbm_entry("expert_gather_kernel, c4", expert_alg_bytes(T, H, k), ms_expert,
+                      "up/down tables (16 MiB) are cache-resident, so algorithmic bytes exceed HBM traffic"),
+            {"kernel": "router stage (linear2 GEMM + BN partial + BN finalize + select), c4", "kernel_ms": ms_router,
+             "algorithmic_flops": 4 * T * H * r},
+        ]
+        # expert kernel at the shape its bandwidth target is quoted on (BASELINE config 3)
+        T3 = 16384
+        x3, up3, down3, g3, i3 = (t.to(dev) for t in oracle.make_expert_inputs(2, T3, H, N, k))
+        ms_e3 = time_call(torch, lambda: hip.hip_omni_expert_func(x3, up3, down3, g3, i3), reps)
+        ms_s3 = time_call(torch, lambda: hip.hip_omni_schedule_func(i3, N), reps)
+        kernels.append(hbm_entry("expert_gather_kernel, c3 (T=16384)", expert_alg_bytes(T3, H, k), ms_e3,
+                                 "up/down tables (16 MiB) are cache-resident, so algorithmic bytes exceed HBM traffic"))
+        kernels.append(hbm_entry("schedule (fill+histogram+scan+scatter, 5 launches), c3", T3 * k * 14 + 8 * (N + 1), ms_s3))
+        out["roofline"] = max(kernels[:3], key=lambda d: d["kernel_ms"])
+        out["roofline_expert"] = kernels[-2]
+        out["kernels"] = kernels
+
     if not a.no_cpu_baseline:
-        # the oracle on the host cores, bounded sample of the same workload
-        n = 2048
+        # the oracle (torch CPU restatement of the reference's PyTorch layer) on the host cores,
+        # on the first 1024 tokens of the same workload, repeated for ~10 s
+        n = 1024
         torch.set_num_threads(min(16, os.cpu_count() or 1))
-        t0 = time.perf_counter()
-        reps = 0
-        while time.perf_counter() - t0 < 10.0:
-            oracle.schedule(ids[:n], N)
-            oracle.expert_forward(x[:n], up, down, gates[:n], ids[:n], compute_dtype=None)
+        xs = x[:, :n].contiguous()
+        reps, t0 = 0, time.perf_counter()
+        while time.perf_counter() - t0 < 10.0 or reps < 2:
+            bx, by = oracle.BNState.fresh(layer.num_expert_sqrt), oracle.BNState.fresh(layer.num_expert_sqrt)
+            oracle.moe_forward(xs, w, bx, by, k, training=True, expert_compute_dtype=None)
             reps += 1
         dt = time.perf_counter() - t0
         out["cpu_baseline"] = {"value": reps * n / dt, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
-                               "sample": f"{reps} x first {n} tokens of the same workload, bf16 torch CPU ops (oracle restatement)"}
+                               "sample": f"{reps} forwards over the first {n} tokens of the same workload, "
+                                         "bf16 torch CPU ops (oracle restatement of OmniMoE_Torch.forward)"}
     print(json.dumps(out))
 
 

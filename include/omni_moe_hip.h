@@ -113,11 +113,17 @@ OMNI_API int32_t omni_mlp_fwd(const void* x, const void* gate_weight, const void
                               const void* residual, void* y, int64_t num_tokens, int32_t hidden_size,
                               int32_t intermediate_size, int32_t dtype, void* workspace, void* stream);
 
-/* Bias-free linear layer  y[T,out] = x[T,in] weight[out,in]^T  on the matrix cores.
- * Replaces the nn.Linear router projections (omni_moe/modules/omni_moe.py:47-52,70-71).
- * in_features a multiple of 8, out_features of 4; dtype bf16 or f16. */
-OMNI_API int32_t omni_linear_fwd(const void* x, const void* weight, void* y, int64_t num_tokens, int32_t in_features,
-                                 int32_t out_features, int32_t dtype, void* stream);
+/* The two halves of omni_mlp_fwd as separate calls.
+ * omni_swiglu_linear_fwd: h[T,I] = silu(x Wg^T) * (x Wu^T)   (interface.py:23-27 + omni_mlp.py:102-177)
+ * omni_linear_fwd:        y[T,out] = x[T,in] weight[out,in]^T [+ residual[T,out]]
+ *                         (a bias-free nn.Linear / torch.matmul(., W.t()): interface.py:23-29,
+ *                          omni_moe/modules/omni_moe.py:47-52,70-71)
+ * in_features / hidden_size multiples of 8, out_features / intermediate_size of 4; bf16 or f16. */
+OMNI_API int32_t omni_swiglu_linear_fwd(const void* x, const void* gate_weight, const void* up_weight, void* h,
+                                        int64_t num_tokens, int32_t hidden_size, int32_t intermediate_size,
+                                        int32_t dtype, void* stream);
+OMNI_API int32_t omni_linear_fwd(const void* x, const void* weight, const void* residual, void* y, int64_t num_tokens,
+                                 int32_t in_features, int32_t out_features, int32_t dtype, void* stream);
 
 /* Two bias-free linear layers sharing their input, written side by side:
  * y[T, 2*out] = [x weight_lo^T | x weight_hi^T].  One GEMM for the router's x and y

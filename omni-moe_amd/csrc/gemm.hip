@@ -309,15 +309,30 @@ extern "C" OMNI_API int32_t omni_mlp_fwd(const void* x, const void* gate_weight,
   }
 }
 
-extern "C" OMNI_API int32_t omni_linear_fwd(const void* x, const void* weight, void* y, int64_t num_tokens, int32_t in_features,
-                                            int32_t out_features, int32_t dtype, void* stream) {
+extern "C" OMNI_API int32_t omni_swiglu_linear_fwd(const void* x, const void* gate_weight, const void* up_weight, void* h,
+                                                   int64_t num_tokens, int32_t hidden_size, int32_t intermediate_size,
+                                                   int32_t dtype, void* stream) {
+  using namespace omni;
+  if (num_tokens == 0) return OMNI_OK;
+  if (!x || !gate_weight || !up_weight || !h) return OMNI_ERR_NULL;
+  hipStream_t s = (hipStream_t)stream;
+  switch (dtype) {
+    case OMNI_BF16: return gemm_swiglu<kBF16>(x, gate_weight, up_weight, h, num_tokens, intermediate_size, hidden_size, s);
+    case OMNI_F16: return gemm_swiglu<kF16>(x, gate_weight, up_weight, h, num_tokens, intermediate_size, hidden_size, s);
+    case OMNI_F32: return OMNI_ERR_UNSUPPORTED;
+    default: return OMNI_ERR_DTYPE;
+  }
+}
+
+extern "C" OMNI_API int32_t omni_linear_fwd(const void* x, const void* weight, const void* residual, void* y, int64_t num_tokens,
+                                            int32_t in_features, int32_t out_features, int32_t dtype, void* stream) {
   using namespace omni;
   if (num_tokens == 0) return OMNI_OK;
   if (!x || !weight || !y) return OMNI_ERR_NULL;
   hipStream_t s = (hipStream_t)stream;
   switch (dtype) {
-    case OMNI_BF16: return gemm_plain<kBF16>(x, weight, nullptr, nullptr, y, num_tokens, out_features, in_features, s);
-    case OMNI_F16: return gemm_plain<kF16>(x, weight, nullptr, nullptr, y, num_tokens, out_features, in_features, s);
+    case OMNI_BF16: return gemm_plain<kBF16>(x, weight, nullptr, residual, y, num_tokens, out_features, in_features, s);
+    case OMNI_F16: return gemm_plain<kF16>(x, weight, nullptr, residual, y, num_tokens, out_features, in_features, s);
     case OMNI_F32: return OMNI_ERR_UNSUPPORTED;
     default: return OMNI_ERR_DTYPE;
   }

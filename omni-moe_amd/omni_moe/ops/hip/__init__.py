@@ -6,7 +6,8 @@ from .interface import (  # noqa: F401
     hip_omni_router_func,
     hip_omni_router_fwd_func,
     hip_omni_schedule_func,
+    hip_swiglu_linear_func,
 )
 
 __all__ = ["hip_omni_router_func", "hip_omni_expert_func", "hip_omni_mlp_func", "hip_omni_schedule_func",
-           "hip_omni_router_fwd_func", "hip_linear_func", "Schedule"]
+           "hip_omni_router_fwd_func", "hip_linear_func", "hip_swiglu_linear_func", "Schedule"]

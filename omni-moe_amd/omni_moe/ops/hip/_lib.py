@@ -32,7 +32,8 @@ SIGNATURES = {
     "omni_expert_workspace_bytes": (c_size_t, [c_int64, c_int32, c_int64, c_int32, c_int32, c_int32]),
     "omni_mlp_workspace_bytes": (c_size_t, [c_int64, c_int32, c_int32, c_int32]),
     "omni_mlp_fwd": (c_int32, [c_void_p] * 6 + [c_int64, c_int32, c_int32, c_int32, c_void_p, c_void_p]),
-    "omni_linear_fwd": (c_int32, [c_void_p] * 3 + [c_int64, c_int32, c_int32, c_int32, c_void_p]),
+    "omni_linear_fwd": (c_int32, [c_void_p] * 4 + [c_int64, c_int32, c_int32, c_int32, c_void_p]),
+    "omni_swiglu_linear_fwd": (c_int32, [c_void_p] * 4 + [c_int64, c_int32, c_int32, c_int32, c_void_p]),
     "omni_linear2_fwd": (c_int32, [c_void_p] * 4 + [c_int64, c_int32, c_int32, c_int32, c_void_p]),
     "omni_router_workspace_bytes": (c_size_t, [c_int64, c_int32, c_int32]),
     "omni_router_fwd": (c_int32, [c_void_p] * 9 + [c_int32, c_float, c_float, c_void_p, c_void_p, c_void_p,

@@ -168,20 +168,40 @@ def hip_omni_mlp_func(
     return y
 
 
-def hip_linear_func(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
-    """x @ weight.T for a bias-free ``nn.Linear`` (the router projections, reference omni_moe.py:70-71)."""
+def hip_linear_func(x: torch.Tensor, weight: torch.Tensor, residual: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x @ weight.T (+ residual) for a bias-free ``nn.Linear`` (reference omni_moe.py:70-71, interface.py:23-29)."""
     if x.dim() != 2 or weight.dim() != 2 or weight.size(1) != x.size(1):
         raise ValueError("expected x (tokens, in) and weight (out, in)")
     if x.dtype not in (torch.bfloat16, torch.float16) or weight.dtype != x.dtype:
         raise TypeError("x and weight must share a dtype in {bfloat16, float16}")
+    if residual is not None and (residual.shape != (x.size(0), weight.size(0)) or residual.dtype != x.dtype):
+        raise ValueError("residual must be (tokens, out) in x's dtype")
     dev = _lib.require_gpu(x, weight)
     x, weight = _c(x), _c(weight)
+    residual = _c(residual) if residual is not None else None
     y = torch.empty((x.size(0), weight.size(0)), device=dev, dtype=x.dtype)
     with torch.cuda.device(dev):
-        code = _lib.load().omni_linear_fwd(_lib.ptr(x), _lib.ptr(weight), _lib.ptr(y), x.size(0), x.size(1), weight.size(0),
-                                           _lib.DTYPE_CODE[x.dtype], _lib.stream_ptr())
+        code = _lib.load().omni_linear_fwd(_lib.ptr(x), _lib.ptr(weight), _lib.ptr(residual), _lib.ptr(y), x.size(0), x.size(1),
+                                           weight.size(0), _lib.DTYPE_CODE[x.dtype], _lib.stream_ptr())
     _lib.check(code, "omni_linear_fwd")
     return y
+
+
+def hip_swiglu_linear_func(x: torch.Tensor, gate_weight: torch.Tensor, up_weight: torch.Tensor) -> torch.Tensor:
+    """silu(x gate^T) * (x up^T): the first half of the MLP op as one GEMM with a fused epilogue."""
+    if x.dim() != 2 or gate_weight.shape != up_weight.shape or gate_weight.dim() != 2 or gate_weight.size(1) != x.size(1):
+        raise ValueError("expected x (tokens, hidden) and gate/up weights (intermediate, hidden)")
+    if x.dtype not in (torch.bfloat16, torch.float16) or gate_weight.dtype != x.dtype or up_weight.dtype != x.dtype:
+        raise TypeError("x and the weights must share a dtype in {bfloat16, float16}")
+    dev = _lib.require_gpu(x, gate_weight, up_weight)
+    x, gate_weight, up_weight = map(_c, (x, gate_weight, up_weight))
+    h = torch.empty((x.size(0), gate_weight.size(0)), device=dev, dtype=x.dtype)
+    with torch.cuda.device(dev):
+        code = _lib.load().omni_swiglu_linear_fwd(_lib.ptr(x), _lib.ptr(gate_weight), _lib.ptr(up_weight), _lib.ptr(h),
+                                                  x.size(0), x.size(1), gate_weight.size(0), _lib.DTYPE_CODE[x.dtype],
+                                                  _lib.stream_ptr())
+    _lib.check(code, "omni_swiglu_linear_fwd")
+    return h
 
 
 def hip_omni_router_fwd_func(
