@@ -49,6 +49,8 @@ struct GemmArgs {
   int M, N, K;            // N = output columns
   int tiles_m, tiles_n;
   int patch_m, patch_n;   // XCD patch shape (0 = plain order)
+  float* part_mean;       // plain epilogue only, may be NULL: [ceil(M/32)][N] mean of each column over
+  float* part_m2;         //   rows 32s..32s+31 of the ROUNDED result, and the sum of squared deviations
 };
 
 // 16-bit storage, TM x TN MFMA tiles per wave.  For the SwiGLU epilogue the first TN/2
@@ -169,6 +171,38 @@ __global__ __launch_bounds__(kGemmThreads, 1) void gemm_nt_kernel(const GemmArgs
     __syncthreads();
   }
 
+  // ---- column statistics of the rounded tile for BatchNorm: every 32-row MFMA tile is one
+  // strip; a column lives in the 32 lanes that share lane/32, so five xor-shuffles reduce it
+  if constexpr (EPI == kEpiPlain) {
+    if (g.part_mean) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        const int row0 = m0 + wm * TM * 32 + i * 32;
+        const int cnt = min(32, g.M - row0);
+        if (cnt <= 0) continue;
+        const bool live = (lane & 31) < cnt;
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+          for (int q = 0; q < 16; ++q) {
+            const float v = live ? Elem<DT>::round(acc[i][j][q]) : 0.f;
+            float sum = v;
+#pragma unroll
+            for (int mk = 16; mk >= 1; mk >>= 1) sum += __shfl_xor(sum, mk, kWave);
+            const float mean = sum / float(cnt);
+            float dev = live ? (v - mean) * (v - mean) : 0.f;
+#pragma unroll
+            for (int mk = 16; mk >= 1; mk >>= 1) dev += __shfl_xor(dev, mk, kWave);
+            const int n = n0 + wn * TN * 32 + j * 32 + (q >> 2) * 8 + (lane >> 5) * 4 + (q & 3);
+            if ((lane & 31) == 0 && n < g.N) {
+              g.part_mean[(int64_t)(row0 >> 5) * g.N + n] = mean;
+              g.part_m2[(int64_t)(row0 >> 5) * g.N + n] = dev;
+            }
+          }
+      }
+    }
+  }
+
   // ---- epilogue.  acc[i][j][q]: row m = lane%32, column n = (q/4)*8 + (lane/32)*4 + q%4
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
@@ -248,10 +282,13 @@ static int to_code(hipError_t e) { return e == hipSuccess ? OMNI_OK : OMNI_ERR_H
 
 // C[M,N] = A[M,K] B[N,K]^T (+ res), picking the tile shape from the problem size.
 template <int DT>
-static int gemm_plain(const void* a, const void* b, const void* b_hi, const void* res, void* c, int64_t M, int64_t N, int64_t K, hipStream_t s) {
+static int gemm_plain(const void* a, const void* b, const void* b_hi, const void* res, void* c, int64_t M, int64_t N, int64_t K, hipStream_t s,
+                      float* part_mean = nullptr, float* part_m2 = nullptr) {
   if (int e = check_gemm(M, N, K)) return e;
   if (M == 0) return OMNI_OK;
-  GemmArgs g{(const uint16_t*)a, (const uint16_t*)b, (const uint16_t*)b_hi, (const uint16_t*)res, (uint16_t*)c, (int)M, (int)N, (int)K, 0, 0, 0, 0};
+  GemmArgs g{(const uint16_t*)a, (const uint16_t*)b, (const uint16_t*)b_hi, (const uint16_t*)res, (uint16_t*)c, (int)M, (int)N, (int)K, 0, 0, 0, 0, nullptr, nullptr};
+  g.part_mean = part_mean;
+  g.part_m2 = part_m2;
   const int64_t big = ((M + 255) / 256) * ((N + 255) / 256), mid = ((M + 127) / 128) * ((N + 127) / 128);
   hipError_t err;
   if (res) {
@@ -270,7 +307,7 @@ template <int DT>
 static int gemm_swiglu(const void* x, const void* wg, const void* wu, void* h, int64_t M, int64_t I, int64_t K, hipStream_t s) {
   if (int e = check_gemm(M, I, K)) return e;
   if (M == 0) return OMNI_OK;
-  GemmArgs g{(const uint16_t*)x, (const uint16_t*)wg, (const uint16_t*)wu, nullptr, (uint16_t*)h, (int)M, (int)I, (int)K, 0, 0, 0, 0};
+  GemmArgs g{(const uint16_t*)x, (const uint16_t*)wg, (const uint16_t*)wu, nullptr, (uint16_t*)h, (int)M, (int)I, (int)K, 0, 0, 0, 0, nullptr, nullptr};
   const int64_t big = ((M + 255) / 256) * ((I + 127) / 128);
   hipError_t err;
   if (big >= 200) err = launch_gemm<DT, 4, 4, kEpiSwiglu>(g, s);
@@ -279,6 +316,15 @@ static int gemm_swiglu(const void* x, const void* wg, const void* wu, void* h, i
 }
 
 }  // namespace omni
+
+int omni_gemm_router_projection(const void* x, const void* wx, const void* wy, void* z, float* part_mean, float* part_m2,
+                                int64_t T, int H, int r, int dtype, void* stream) {
+  using namespace omni;
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == OMNI_BF16) return gemm_plain<kBF16>(x, wx, wy, nullptr, z, T, 2 * (int64_t)r, H, s, part_mean, part_m2);
+  if (dtype == OMNI_F16) return gemm_plain<kF16>(x, wx, wy, nullptr, z, T, 2 * (int64_t)r, H, s, part_mean, part_m2);
+  return OMNI_ERR_UNSUPPORTED;
+}
 
 extern "C" OMNI_API size_t omni_mlp_workspace_bytes(int64_t num_tokens, int32_t hidden_size, int32_t intermediate_size, int32_t dtype) {
   (void)hidden_size;

@@ -17,6 +17,11 @@
 #include "common.h"
 #include "omni_moe_hip.h"
 
+// defined beside the GEMM kernels: z = x [Wx;Wy]^T, optionally with per-32-row column
+// partial statistics (mean, M2) [ceil(T/32)][2r] of the rounded z
+int omni_gemm_router_projection(const void* x, const void* wx, const void* wy, void* z, float* part_mean, float* part_m2,
+                                int64_t T, int H, int r, int dtype, void* stream);
+
 namespace omni {
 
 // strict "a goes before b": higher score first, then lower payload
@@ -88,6 +93,34 @@ __device__ __forceinline__ void bitonic_sort(float (&s)[R], int (&p)[R], const i
     for (int stride = size >> 1; stride >= 1; stride >>= 1) lane_stage<R>(s, p, lane, size, stride);
   }
   big_sizes<R, 2 * kWave>(s, p, lane);
+}
+
+// Two independent lists sorted in lockstep: the two dependency chains interleave, which
+// hides most of the cross-lane exchange latency.
+template <int R, int SIZE>
+__device__ __forceinline__ void big_sizes2(float (&s0)[R], int (&p0)[R], float (&s1)[R], int (&p1)[R], const int lane) {
+  if constexpr (SIZE <= kWave * R) {
+    reg_stages_down<R, SIZE, SIZE / (2 * kWave)>(s0, p0);
+    reg_stages_down<R, SIZE, SIZE / (2 * kWave)>(s1, p1);
+#pragma nounroll
+    for (int stride = kWave / 2; stride >= 1; stride >>= 1) {
+      lane_stage<R>(s0, p0, lane, SIZE, stride);
+      lane_stage<R>(s1, p1, lane, SIZE, stride);
+    }
+    big_sizes2<R, SIZE * 2>(s0, p0, s1, p1, lane);
+  }
+}
+template <int R>
+__device__ __forceinline__ void bitonic_sort2(float (&s0)[R], int (&p0)[R], float (&s1)[R], int (&p1)[R], const int lane) {
+#pragma nounroll
+  for (int size = 2; size <= kWave; size <<= 1) {
+#pragma nounroll
+    for (int stride = size >> 1; stride >= 1; stride >>= 1) {
+      lane_stage<R>(s0, p0, lane, size, stride);
+      lane_stage<R>(s1, p1, lane, size, stride);
+    }
+  }
+  big_sizes2<R, 2 * kWave>(s0, p0, s1, p1, lane);
 }
 
 // value of sorted item `i` (i < 128) of a list held as item = reg*64+lane
@@ -189,8 +222,7 @@ __global__ __launch_bounds__(kRouterWaves* kWave) void router_select_kernel(cons
       normalise_half<R>(sx, g.stats, g.stats + r, r, lane, dt);
       normalise_half<R>(sy, g.stats + 2 * r, g.stats + 3 * r, r, lane, dt);
     }
-    bitonic_sort<R>(sx, px, lane);
-    bitonic_sort<R>(sy, py, lane);
+    bitonic_sort2<R>(sx, px, sy, py, lane);
 
     float cs[C];
     int cp[C];
@@ -259,31 +291,7 @@ static int select_dispatch(SelectArgs g, hipStream_t s) {
 }
 
 // ---- BatchNorm1d(affine=False) statistics over the T rows of z [T, C] -------------------
-constexpr int kBnRows = 32;       // rows per partial
-
-// Partial (mean, M2) of every column over a strip of <= 32 rows, two passes over registers.
-__global__ __launch_bounds__(256) void bn_partial_kernel(const void* __restrict__ z, float* __restrict__ part_mean,
-                                                         float* __restrict__ part_m2, int num_rows, int num_cols, int dt) {
-  const int col = blockIdx.x * 256 + threadIdx.x;
-  if (col >= num_cols) return;
-  const int row0 = blockIdx.y * kBnRows;
-  const int n = min(kBnRows, num_rows - row0);
-  float v[kBnRows], sum = 0.f;
-#pragma unroll
-  for (int i = 0; i < kBnRows; ++i) {
-    v[i] = (i < n) ? load_score(z, int64_t(row0 + i) * num_cols + col, dt) : 0.f;
-    sum += v[i];
-  }
-  const float mean = sum / float(n);
-  float m2 = 0.f;
-#pragma unroll
-  for (int i = 0; i < kBnRows; ++i) {
-    const float d = v[i] - mean;
-    m2 += (i < n) ? d * d : 0.f;
-  }
-  part_mean[int64_t(blockIdx.y) * num_cols + col] = mean;
-  part_m2[int64_t(blockIdx.y) * num_cols + col] = m2;
-}
+constexpr int kBnRows = 32;       // rows per partial: one 32-row MFMA tile of the projection GEMM
 
 struct BnFinalArgs {
   const float* part_mean;   // [strips][2r] (training)
@@ -296,12 +304,19 @@ struct BnFinalArgs {
   float momentum, eps;
 };
 
-// One thread per column: merges the strip partials (Chan's update, in double), writes mean
-// and 1/sqrt(var+eps), and in training moves the running buffers (unbiased variance) as
-// nn.BatchNorm1d does.  In eval the running buffers provide mean and variance.
+__device__ __forceinline__ double wave_sum_f64(double v) {
+#pragma unroll
+  for (int m = kWave / 2; m >= 1; m >>= 1) v += __shfl_xor(v, m, kWave);
+  return v;
+}
+
+// One wave per column: merges the strip partials exactly (mean = sum n_s mean_s / n,
+// M2 = sum M2_s + n_s (mean_s - mean)^2, in double), writes mean and 1/sqrt(var+eps), and in
+// training moves the running buffers (unbiased variance) as nn.BatchNorm1d does.  In eval
+// the running buffers provide mean and variance.
 __global__ __launch_bounds__(256) void bn_finalize_kernel(const BnFinalArgs g) {
-  const int col = blockIdx.x * 256 + threadIdx.x;
-  if (col == 0 && g.training) {
+  const int col = blockIdx.x * (256 / kWave) + (threadIdx.x >> 6), lane = lane_id();
+  if (col == 0 && lane == 0 && g.training) {
     if (g.num_batches_tracked[0]) *g.num_batches_tracked[0] += 1;
     if (g.num_batches_tracked[1]) *g.num_batches_tracked[1] += 1;
   }
@@ -309,27 +324,32 @@ __global__ __launch_bounds__(256) void bn_finalize_kernel(const BnFinalArgs g) {
   const int half = col >= g.r, key = col - half * g.r;
   float mean, var;
   if (g.training) {
-    double n = 0., mu = 0., m2 = 0.;
-    for (int s = 0; s < g.strips; ++s) {
-      const double nb = (double)min(kBnRows, g.num_rows - s * kBnRows);
-      const double mb = g.part_mean[int64_t(s) * 2 * g.r + col], qb = g.part_m2[int64_t(s) * 2 * g.r + col];
-      const double d = mb - mu, nn = n + nb;
-      mu += d * nb / nn;
-      m2 += qb + d * d * n * nb / nn;
-      n = nn;
+    double wsum = 0.;
+    for (int s = lane; s < g.strips; s += kWave)
+      wsum += (double)min(kBnRows, g.num_rows - s * kBnRows) * (double)g.part_mean[int64_t(s) * 2 * g.r + col];
+    const double n = (double)g.num_rows, mu = wave_sum_f64(wsum) / n;
+    double q = 0.;
+    for (int s = lane; s < g.strips; s += kWave) {
+      const double d = (double)g.part_mean[int64_t(s) * 2 * g.r + col] - mu;
+      q += (double)g.part_m2[int64_t(s) * 2 * g.r + col] + (double)min(kBnRows, g.num_rows - s * kBnRows) * d * d;
     }
+    const double m2 = wave_sum_f64(q);
     mean = (float)mu;
     var = (float)(m2 / n);                                   // biased: normalises the batch
-    const float unbiased = (float)(m2 / (n > 1. ? n - 1. : 1.));
-    const float rm = load_score(g.running_mean[half], key, g.stat_dt), rv = load_score(g.running_var[half], key, g.stat_dt);
-    store_score(g.running_mean[half], key, (1.f - g.momentum) * rm + g.momentum * mean, g.stat_dt);
-    store_score(g.running_var[half], key, (1.f - g.momentum) * rv + g.momentum * unbiased, g.stat_dt);
+    if (lane == 0) {
+      const float unbiased = (float)(m2 / (n > 1. ? n - 1. : 1.));
+      const float rm = load_score(g.running_mean[half], key, g.stat_dt), rv = load_score(g.running_var[half], key, g.stat_dt);
+      store_score(g.running_mean[half], key, (1.f - g.momentum) * rm + g.momentum * mean, g.stat_dt);
+      store_score(g.running_var[half], key, (1.f - g.momentum) * rv + g.momentum * unbiased, g.stat_dt);
+    }
   } else {
     mean = load_score(g.running_mean[half], key, g.stat_dt);
     var = load_score(g.running_var[half], key, g.stat_dt);
   }
-  g.stats[(2 * half) * g.r + key] = mean;
-  g.stats[(2 * half + 1) * g.r + key] = 1.0f / sqrtf(var + g.eps);
+  if (lane == 0) {
+    g.stats[(2 * half) * g.r + key] = mean;
+    g.stats[(2 * half + 1) * g.r + key] = 1.0f / sqrtf(var + g.eps);
+  }
 }
 
 static inline size_t align256(size_t v) { return (v + 255) / 256 * 256; }
@@ -385,14 +405,13 @@ extern "C" OMNI_API int32_t omni_router_fwd(const void* x, const void* weight_x,
   float* part_m2 = (float*)w;
 
   // z = x [Wx;Wy]^T on the matrix cores
-  if (int e = omni_linear2_fwd(x, weight_x, weight_y, z, num_tokens, hidden_size, r, dtype, stream)) return e;
-  if (training)
-    hipLaunchKernelGGL(bn_partial_kernel, dim3((2 * r + 255) / 256, (unsigned)strips), dim3(256), 0, s, z, part_mean, part_m2,
-                       (int)num_tokens, 2 * r, dtype);
+  // (in training its epilogue also leaves the per-32-row column statistics)
+  if (int e = omni_gemm_router_projection(x, weight_x, weight_y, z, training ? part_mean : nullptr, training ? part_m2 : nullptr,
+                                          num_tokens, hidden_size, r, dtype, stream)) return e;
   BnFinalArgs b{part_mean, part_m2, stats, {running_mean_x, running_mean_y}, {running_var_x, running_var_y},
                 {num_batches_tracked_x, num_batches_tracked_y}, (int)num_tokens, r, (int)strips, training ? 1 : 0, stats_dtype,
                 momentum, eps};
-  hipLaunchKernelGGL(bn_finalize_kernel, dim3((2 * r + 255) / 256), dim3(256), 0, s, b);
+  hipLaunchKernelGGL(bn_finalize_kernel, dim3((2 * r + 3) / 4), dim3(256), 0, s, b);
   hipError_t err = hipGetLastError();
   if (err != hipSuccess) return OMNI_ERR_HIP_BASE + (int)err;
   if (k == 0) return OMNI_OK;
