@@ -16,6 +16,13 @@
 
 namespace omni {
 
+#ifdef OMNI_GEMM_TIMING
+__device__ long long* g_timing = nullptr;   // [blocks][8] cycle stamps, debug builds only
+#define OMNI_STAMP(slot) do { if (g_timing && threadIdx.x == 0) g_timing[blockIdx.x * 8 + (slot)] = (long long)__builtin_readcyclecounter(); } while (0)
+#else
+#define OMNI_STAMP(slot) do { } while (0)
+#endif
+
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
@@ -53,6 +60,105 @@ struct GemmArgs {
   float* part_m2;         //   rows 32s..32s+31 of the ROUNDED result, and the sum of squared deviations
 };
 
+// Which output tile a block owns.  Blocks go round-robin over the 8 XCDs; each XCD gets
+// compact patches of tiles so that the blocks sharing its L2 share operand panels.
+__device__ __forceinline__ void tile_coords(const GemmArgs& g, int& tile_m, int& tile_n) {
+  const int b = blockIdx.x;
+  if (g.patch_m > 0) {
+    const int per_patch = g.patch_m * g.patch_n;
+    const int xcd = b & 7, idx = b >> 3;
+    const int patch = (idx / per_patch) * 8 + xcd, within = idx % per_patch;
+    const int patches_m = g.tiles_m / g.patch_m;
+    tile_m = (patch % patches_m) * g.patch_m + within % g.patch_m;
+    tile_n = (patch / patches_m) * g.patch_n + within / g.patch_m;
+  } else {
+    tile_m = b % g.tiles_m;
+    tile_n = b / g.tiles_m;
+  }
+}
+
+// Writes a wave's TM x TN accumulator tiles.  acc[i][j][q] is row m = lane%32 and column
+// n = (q/4)*8 + (lane/32)*4 + q%4 of MFMA tile (i, j).
+template <int DT, int TM, int TN, int EPI>
+__device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, f32x16_t (&acc)[TM][TN], const int m0, const int n0,
+                                              const int wm, const int wn, const int lane) {
+  constexpr int TNO = (EPI == kEpiSwiglu) ? TN / 2 : TN;
+  // ---- column statistics of the rounded tile for BatchNorm: every 32-row MFMA tile is one
+  // strip; a column lives in the 32 lanes that share lane/32, so five xor-shuffles reduce it
+  if constexpr (EPI == kEpiPlain) {
+    if (g.part_mean) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        const int row0 = m0 + wm * TM * 32 + i * 32;
+        const int cnt = min(32, g.M - row0);
+        if (cnt <= 0) continue;
+        const bool live = (lane & 31) < cnt;
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+          for (int q = 0; q < 16; ++q) {
+            const float v = live ? Elem<DT>::round(acc[i][j][q]) : 0.f;
+            float sum = v;
+#pragma unroll
+            for (int mk = 16; mk >= 1; mk >>= 1) sum += __shfl_xor(sum, mk, kWave);
+            const float mean = sum / float(cnt);
+            float dev = live ? (v - mean) * (v - mean) : 0.f;
+#pragma unroll
+            for (int mk = 16; mk >= 1; mk >>= 1) dev += __shfl_xor(dev, mk, kWave);
+            const int n = n0 + wn * TN * 32 + j * 32 + (q >> 2) * 8 + (lane >> 5) * 4 + (q & 3);
+            if ((lane & 31) == 0 && n < g.N) {
+              g.part_mean[(int64_t)(row0 >> 5) * g.N + n] = mean;
+              g.part_m2[(int64_t)(row0 >> 5) * g.N + n] = dev;
+            }
+          }
+      }
+    }
+  }
+
+  // ---- epilogue.  acc[i][j][q]: row m = lane%32, column n = (q/4)*8 + (lane/32)*4 + q%4
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    const int m = m0 + wm * TM * 32 + i * 32 + (lane & 31);
+    if (m >= g.M) continue;
+#pragma unroll
+    for (int j = 0; j < TNO; ++j) {
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        const int n = n0 + wn * TNO * 32 + j * 32 + q4 * 8 + (lane >> 5) * 4;
+        if (n >= g.N) continue;                          // N is a multiple of 4
+        float v[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          if constexpr (EPI == kEpiSwiglu) {
+            // the reference materialises gate and up in the storage dtype, then forms
+            // silu(gate)*up in fp32 and rounds once (omni_mlp.py:53-61)
+            const float gt = Elem<DT>::round(acc[i][j][q4 * 4 + q]);
+            const float up = Elem<DT>::round(acc[i][j + TNO][q4 * 4 + q]);
+            v[q] = silu_fast(gt) * up;
+          } else {
+            v[q] = acc[i][j][q4 * 4 + q];
+          }
+        }
+        const int64_t o = (int64_t)m * g.N + n;
+        if constexpr (EPI == kEpiResidual) {
+          // y = round(h Wd^T) + e, rounded again: the reference adds two stored tensors
+          const u32x2_t r = *(const u32x2_t*)(g.res + o);
+          const uint32_t r0 = r[0], r1 = r[1];
+          if constexpr (DT == kBF16) {
+            v[0] = Elem<DT>::round(v[0]) + bf16_lo(r0); v[1] = Elem<DT>::round(v[1]) + bf16_hi(r0);
+            v[2] = Elem<DT>::round(v[2]) + bf16_lo(r1); v[3] = Elem<DT>::round(v[3]) + bf16_hi(r1);
+          } else {
+            v[0] = Elem<DT>::round(v[0]) + f16_bits_to_f32(r0 & 0xffff); v[1] = Elem<DT>::round(v[1]) + f16_bits_to_f32(r0 >> 16);
+            v[2] = Elem<DT>::round(v[2]) + f16_bits_to_f32(r1 & 0xffff); v[3] = Elem<DT>::round(v[3]) + f16_bits_to_f32(r1 >> 16);
+          }
+        }
+        u32x2_t w = {pack2<DT>(v[0], v[1]), pack2<DT>(v[2], v[3])};
+        *(u32x2_t*)(g.c + o) = w;
+      }
+    }
+  }
+}
+
 // 16-bit storage, TM x TN MFMA tiles per wave.  For the SwiGLU epilogue the first TN/2
 // tiles of a wave are gate columns and the last TN/2 the matching up columns.
 template <int DT, int TM, int TN, int EPI>
@@ -67,23 +173,8 @@ __global__ __launch_bounds__(kGemmThreads, 1) void gemm_nt_kernel(const GemmArgs
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave & 1, wn = wave >> 1;
 
-  // ---- which tile: blocks go round-robin over the 8 XCDs; give each XCD compact
-  // patches of tiles so that the blocks sharing its L2 share operand panels
   int tile_m, tile_n;
-  {
-    const int b = blockIdx.x;
-    if (g.patch_m > 0) {
-      const int per_patch = g.patch_m * g.patch_n;
-      const int xcd = b & 7, idx = b >> 3;
-      const int patch = (idx / per_patch) * 8 + xcd, within = idx % per_patch;
-      const int patches_m = g.tiles_m / g.patch_m;
-      tile_m = (patch % patches_m) * g.patch_m + within % g.patch_m;
-      tile_n = (patch / patches_m) * g.patch_n + within / g.patch_m;
-    } else {
-      tile_m = b % g.tiles_m;
-      tile_n = b / g.tiles_m;
-    }
-  }
+  tile_coords(g, tile_m, tile_n);
   const int m0 = tile_m * BM, n0 = tile_n * BN;
 
   // ---- global -> register staging: thread owns 16-byte chunk (tid%8) of rows tid/8 + 32*p
@@ -171,80 +262,177 @@ __global__ __launch_bounds__(kGemmThreads, 1) void gemm_nt_kernel(const GemmArgs
     __syncthreads();
   }
 
-  // ---- column statistics of the rounded tile for BatchNorm: every 32-row MFMA tile is one
-  // strip; a column lives in the 32 lanes that share lane/32, so five xor-shuffles reduce it
-  if constexpr (EPI == kEpiPlain) {
-    if (g.part_mean) {
+  gemm_epilogue<DT, TM, TN, EPI>(g, acc, m0, n0, wm, wn, lane);
+}
+
+// ---- main kernel: global -> LDS without passing through registers ------------------------
+// K advances BK (32 or 64) at a time through a ring of NS LDS stages that
+// `global_load_lds_dwordx4` fills directly.  Each wave instruction lands 1 KiB of consecutive
+// LDS, so rows cannot be padded; instead the 16-byte chunk c of row r is kept at a swizzled
+// chunk position (the loading lane applies the swizzle to its GLOBAL address), chosen so that
+// the 128-bit fragment reads of 16 consecutive rows cover all 64 banks once.  NS-2 tiles are
+// in flight while one is computed.  The K=16 slabs are skewed across the tile boundary: the
+// last slab's fragments of a tile are in registers before the barrier that releases its
+// stage, so the MFMAs of one slab always cover the LDS reads of the next.  Needs K % BK == 0.
+template <int N> __device__ __forceinline__ void wait_vmcnt() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
+__device__ __forceinline__ void wait_lds_reads() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+
+// chunk position of logical 16-byte chunk c in row r of a tile whose rows hold BK elements
+template <int BK> __device__ __forceinline__ int swizzle(int r, int c) {
+  if constexpr (BK == 32) return c ^ ((r >> 2) & 3);      // 4 chunks per 64-byte row
+  else return c ^ ((r >> 1) & 7);                          // 8 chunks per 128-byte row
+}
+
+template <int DT, int TM, int TN, int EPI, int BK, int NS>
+__global__ __launch_bounds__(kGemmThreads, 1) void gemm_nt_dma_kernel(const GemmArgs g) {
+  constexpr int BM = 2 * TM * 32, BR = 2 * TN * 32;
+  constexpr int BN = (EPI == kEpiSwiglu) ? BR / 2 : BR;
+  constexpr int TNO = (EPI == kEpiSwiglu) ? TN / 2 : TN;
+  constexpr int kRow = BK * 2;                         // bytes per LDS row
+  constexpr int kCpr = kRow / 16;                      // chunks per row
+  constexpr int kRpi = 64 / kCpr;                      // rows one wave instruction fills
+  constexpr int kStageBytes = (BM + BR) * kRow;
+  constexpr int PA = BM / (4 * kRpi), PB = BR / (4 * kRpi);   // load instructions per wave per tile
+  constexpr int LPT = PA + PB;
+  constexpr int S = BK / 16;                           // slabs per tile
+  extern __shared__ __align__(16) uint8_t lds[];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave & 1, wn = wave >> 1;
+  int tile_m, tile_n;
+  tile_coords(g, tile_m, tile_n);
+#ifdef OMNI_GEMM_SAME_TILE
+  tile_m &= 1; tile_n &= 1;   // debug: every block works on one of 4 tiles (operands stay in L2)
+#endif
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+  // load instruction p of wave w fills tile rows (4p+w)*kRpi ..: lane -> row lane/kCpr, position lane%kCpr
+  const uint8_t* a_src[PA];
+  const uint8_t* b_src[PB];
 #pragma unroll
-      for (int i = 0; i < TM; ++i) {
-        const int row0 = m0 + wm * TM * 32 + i * 32;
-        const int cnt = min(32, g.M - row0);
-        if (cnt <= 0) continue;
-        const bool live = (lane & 31) < cnt;
+  for (int p = 0; p < PA; ++p) {
+    const int rl = (4 * p + wave) * kRpi + lane / kCpr;
+    const int c = swizzle<BK>(rl, lane % kCpr);        // an involution: position -> logical chunk
+    int row = m0 + rl;
+    row = row < g.M ? row : g.M - 1;                    // clamp: tail rows are never stored
+    a_src[p] = (const uint8_t*)(g.a + (int64_t)row * g.K + c * 8);
+  }
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
-#pragma unroll
-          for (int q = 0; q < 16; ++q) {
-            const float v = live ? Elem<DT>::round(acc[i][j][q]) : 0.f;
-            float sum = v;
-#pragma unroll
-            for (int mk = 16; mk >= 1; mk >>= 1) sum += __shfl_xor(sum, mk, kWave);
-            const float mean = sum / float(cnt);
-            float dev = live ? (v - mean) * (v - mean) : 0.f;
-#pragma unroll
-            for (int mk = 16; mk >= 1; mk >>= 1) dev += __shfl_xor(dev, mk, kWave);
-            const int n = n0 + wn * TN * 32 + j * 32 + (q >> 2) * 8 + (lane >> 5) * 4 + (q & 3);
-            if ((lane & 31) == 0 && n < g.N) {
-              g.part_mean[(int64_t)(row0 >> 5) * g.N + n] = mean;
-              g.part_m2[(int64_t)(row0 >> 5) * g.N + n] = dev;
-            }
-          }
-      }
+  for (int p = 0; p < PB; ++p) {
+    const int rl = (4 * p + wave) * kRpi + lane / kCpr;   // row of the weight tile in LDS
+    const int c = swizzle<BK>(rl, lane % kCpr);
+    const uint16_t* base = g.b0;
+    int col;
+    if constexpr (EPI == kEpiSwiglu) {
+      const int pw = rl / (TN * 32), pj = (rl >> 5) % TN;
+      base = (pj < TNO) ? g.b0 : g.b1;
+      col = n0 + pw * (TNO * 32) + (pj % TNO) * 32 + (rl & 31);
+    } else {
+      col = n0 + rl;
     }
+    col = col < g.N ? col : g.N - 1;
+    if constexpr (EPI == kEpiPlain) {
+      if (g.b1 && col >= g.N / 2) { base = g.b1; col -= g.N / 2; }
+    }
+    b_src[p] = (const uint8_t*)(base + (int64_t)col * g.K + c * 8);
   }
 
-  // ---- epilogue.  acc[i][j][q]: row m = lane%32, column n = (q/4)*8 + (lane/32)*4 + q%4
+  auto issue_tile = [&](int kt) {
+    uint8_t* st = lds + (kt % NS) * kStageBytes;
+    const int koff = kt * kRow;
 #pragma unroll
-  for (int i = 0; i < TM; ++i) {
-    const int m = m0 + wm * TM * 32 + i * 32 + (lane & 31);
-    if (m >= g.M) continue;
+    for (int p = 0; p < PA; ++p)
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(a_src[p] + koff),
+                                       (__attribute__((address_space(3))) void*)(st + (4 * p + wave) * 1024), 16, 0, 0);
 #pragma unroll
-    for (int j = 0; j < TNO; ++j) {
+    for (int p = 0; p < PB; ++p)
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(b_src[p] + koff),
+                                       (__attribute__((address_space(3))) void*)(st + BM * kRow + (4 * p + wave) * 1024), 16, 0, 0);
+  };
+
+  // fragment reads: lane reads row lane%32, logical chunk 2*slab + lane/32, into buffer slab&1
+  const int rl = lane & 31;
+  int off_slab[S];
 #pragma unroll
-      for (int q4 = 0; q4 < 4; ++q4) {
-        const int n = n0 + wn * TNO * 32 + j * 32 + q4 * 8 + (lane >> 5) * 4;
-        if (n >= g.N) continue;                          // N is a multiple of 4
-        float v[4];
+  for (int sl = 0; sl < S; ++sl) off_slab[sl] = rl * kRow + swizzle<BK>(rl, 2 * sl + (lane >> 5)) * 16;
+  const int a_frag = (wm * TM * 32) * kRow, b_frag = BM * kRow + (wn * TN * 32) * kRow;
+  u32x4_t af[2][TM], bf[2][TN];
+  auto read_frags = [&](int kt, int slab) {
+    const uint8_t* st = lds + (kt % NS) * kStageBytes + off_slab[slab];
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          if constexpr (EPI == kEpiSwiglu) {
-            // the reference materialises gate and up in the storage dtype, then forms
-            // silu(gate)*up in fp32 and rounds once (omni_mlp.py:53-61)
-            const float gt = Elem<DT>::round(acc[i][j][q4 * 4 + q]);
-            const float up = Elem<DT>::round(acc[i][j + TNO][q4 * 4 + q]);
-            v[q] = silu_f32(gt) * up;
-          } else {
-            v[q] = acc[i][j][q4 * 4 + q];
-          }
-        }
-        const int64_t o = (int64_t)m * g.N + n;
-        if constexpr (EPI == kEpiResidual) {
-          // y = round(h Wd^T) + e, rounded again: the reference adds two stored tensors
-          const u32x2_t r = *(const u32x2_t*)(g.res + o);
-          const uint32_t r0 = r[0], r1 = r[1];
-          if constexpr (DT == kBF16) {
-            v[0] = Elem<DT>::round(v[0]) + bf16_lo(r0); v[1] = Elem<DT>::round(v[1]) + bf16_hi(r0);
-            v[2] = Elem<DT>::round(v[2]) + bf16_lo(r1); v[3] = Elem<DT>::round(v[3]) + bf16_hi(r1);
-          } else {
-            v[0] = Elem<DT>::round(v[0]) + f16_bits_to_f32(r0 & 0xffff); v[1] = Elem<DT>::round(v[1]) + f16_bits_to_f32(r0 >> 16);
-            v[2] = Elem<DT>::round(v[2]) + f16_bits_to_f32(r1 & 0xffff); v[3] = Elem<DT>::round(v[3]) + f16_bits_to_f32(r1 >> 16);
-          }
-        }
-        u32x2_t w = {pack2<DT>(v[0], v[1]), pack2<DT>(v[2], v[3])};
-        *(u32x2_t*)(g.c + o) = w;
-      }
+    for (int i = 0; i < TM; ++i) af[slab & 1][i] = *(const u32x4_t*)(st + a_frag + i * 32 * kRow);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) bf[slab & 1][j] = *(const u32x4_t*)(st + b_frag + j * 32 * kRow);
+  };
+
+  f32x16_t acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int q = 0; q < 16; ++q) acc[i][j][q] = 0.f;
+  // half of a slab's MFMAs (tiles with linear index in [h, h+1) * TM*TN/2), operands in buffer b
+  auto mfma_half = [&](int b, int h) {
+#pragma unroll
+    for (int ij = 0; ij < TM * TN; ++ij) {
+      if ((ij * 2) / (TM * TN) != h) continue;
+      const int i = ij / TN, j = ij % TN;
+      acc[i][j] = mfma32<DT>(bf[b][j], af[b][i], acc[i][j]);
     }
+  };
+  // slab `sl` of a tile while the fragments of the following slab are fetched.  The reads are
+  // issued in the MIDDLE of the slab's MFMAs: the wait the compiler places in front of every
+  // MFMA group covers all LDS reads, so they must be old by the time the next group starts.
+  auto slab_then_read = [&](int sl, int next_kt, int next_slab) {
+    mfma_half(sl & 1, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    read_frags(next_kt, next_slab);
+    __builtin_amdgcn_sched_barrier(0);
+    mfma_half(sl & 1, 1);
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  const int num_kt = g.K / BK;
+  OMNI_STAMP(0);
+#pragma unroll
+  for (int t = 0; t < NS; ++t)
+    if (t < num_kt) issue_tile(t);
+  // before a tile is used, at most NS-2 younger tiles may still be in flight
+  auto wait_tile = [&](int younger) {        // younger = tiles issued after the one needed
+    if constexpr (NS >= 4) { if (younger >= 2) { wait_vmcnt<2 * LPT>(); return; } }
+    if constexpr (NS >= 3) { if (younger >= 1) { wait_vmcnt<LPT>(); return; } }
+    wait_vmcnt<0>();
+  };
+  wait_tile(min(NS, num_kt) - 1 < NS - 2 ? min(NS, num_kt) - 1 : NS - 2);
+  __builtin_amdgcn_s_barrier();
+  OMNI_STAMP(1);
+  read_frags(0, 0);
+  for (int kt = 0; kt < num_kt - 1; ++kt) {
+#pragma unroll
+    for (int sl = 0; sl < S - 1; ++sl) slab_then_read(sl, kt, sl + 1);
+    wait_lds_reads();                         // this wave holds every fragment of tile kt
+    // tiles kt+1 .. min(kt+NS-1, num_kt-1) are outstanding; tile kt+1 must have landed
+    const int younger = num_kt - 2 - kt;
+#ifndef OMNI_DBG_NO_DMA
+    wait_tile(younger < NS - 2 ? younger : NS - 2);
+#endif
+#ifndef OMNI_DBG_NO_BARRIER
+    __builtin_amdgcn_s_barrier();             // tile kt+1 visible to all; stage of tile kt free
+#endif
+#ifndef OMNI_DBG_NO_DMA
+    if (kt + NS < num_kt) issue_tile(kt + NS);
+#endif
+    __builtin_amdgcn_sched_barrier(0);
+    slab_then_read(S - 1, kt + 1, 0);
   }
+#pragma unroll
+  for (int sl = 0; sl < S - 1; ++sl) slab_then_read(sl, num_kt - 1, sl + 1);   // last tile
+  mfma_half((S - 1) & 1, 0);
+  mfma_half((S - 1) & 1, 1);
+  OMNI_STAMP(2);
+  gemm_epilogue<DT, TM, TN, EPI>(g, acc, m0, n0, wm, wn, lane);
+  OMNI_STAMP(3);
 }
 
 template <int DT, int TM, int TN, int EPI>
@@ -260,8 +448,25 @@ static hipError_t launch_gemm(GemmArgs g, hipStream_t s) {
     if (g.tiles_m % 4 == 0 && g.tiles_n % 8 == 0) { g.patch_m = 4; g.patch_n = 8; }
     else if (g.tiles_m % 8 == 0 && g.tiles_n % 4 == 0) { g.patch_m = 8; g.patch_n = 4; }
   }
-  auto kern = gemm_nt_kernel<DT, TM, TN, EPI>;
-  static bool configured = false;                    // idempotent attribute, set once per instantiation
+  // 128-byte LDS rows (64-byte rows halve the fetch rate); as many ring stages as 160 KiB hold, up to 4
+  constexpr int kDmaBK = 64;
+  constexpr int kFit = (160 * 1024) / ((BM + BR) * kDmaBK * 2);
+  constexpr int kDmaStages = kFit > 4 ? 4 : kFit;
+  if (g.K % kDmaBK == 0) {
+    constexpr int kDmaLds = kDmaStages * (BM + BR) * kDmaBK * 2;
+    static_assert(kDmaLds <= 160 * 1024, "LDS ring exceeds 160 KiB");
+    auto kern = gemm_nt_dma_kernel<DT, TM, TN, EPI, kDmaBK, kDmaStages>;
+    static bool configured = false;                  // idempotent attribute, set once per instantiation
+    if (!configured) {
+      hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kDmaLds);
+      if (e != hipSuccess) return e;
+      configured = true;
+    }
+    hipLaunchKernelGGL(kern, dim3(blocks), dim3(kGemmThreads), kDmaLds, s, g);
+    return hipGetLastError();
+  }
+  auto kern = gemm_nt_kernel<DT, TM, TN, EPI>;       // any K % 8 == 0: staged through registers
+  static bool configured = false;
   if (!configured) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
     if (e != hipSuccess) return e;
@@ -399,3 +604,9 @@ extern "C" OMNI_API int32_t omni_linear2_fwd(const void* x, const void* weight_l
     default: return OMNI_ERR_DTYPE;
   }
 }
+
+#ifdef OMNI_GEMM_TIMING
+extern "C" OMNI_API int32_t omni_debug_set_timing(long long* buf) {
+  return (int32_t)hipMemcpyToSymbol(HIP_SYMBOL(omni::g_timing), &buf, sizeof(buf));
+}
+#endif
