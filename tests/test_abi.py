@@ -1,0 +1,101 @@
+"""The C-ABI library loads without a GPU and exports exactly what include/omni_moe_hip.h declares.
+No compute call is made here."""
+import ctypes
+import os
+import re
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "omni_moe_hip.h")
+
+
+def _declared():
+    text = open(HEADER).read()
+    return sorted(set(re.findall(r"OMNI_API\s+[\w\s\*]+?\b(omni_\w+)\s*\(", text)))
+
+
+def _lib():
+    from omni_moe.ops.hip import _lib
+    if not os.path.exists(_lib.LIB_PATH):
+        from omni_moe.ops.hip import build
+        build.build_library()
+    return _lib
+
+
+def test_header_declares_the_path():
+    names = _declared()
+    for must in ("omni_router_select", "omni_router_fwd", "omni_schedule", "omni_expert_fwd", "omni_mlp_fwd"):
+        assert must in names
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib().load()
+    for name in _declared():
+        assert hasattr(lib, name), f"{name} declared in the header but not exported"
+    assert lib.omni_abi_version() == 1
+    assert b"ok" == lib.omni_error_string(0)
+    assert b"NULL" in lib.omni_error_string(-1)
+
+
+def test_binding_table_matches_header():
+    lib = _lib()
+    assert sorted(lib.SIGNATURES) == _declared()
+    # argument counts of the ctypes table equal the header's parameter counts
+    text = re.sub(r"/\*.*?\*/", "", open(HEADER).read(), flags=re.S)
+    for name, (_, args) in lib.SIGNATURES.items():
+        m = re.search(r"\b%s\s*\(([^;]*?)\)\s*;" % name, text, flags=re.S)
+        params = [p for p in m.group(1).split(",") if p.strip() and p.strip() != "void"]
+        assert len(params) == len(args), name
+
+
+def test_no_extra_exports():
+    lib = _lib()
+    out = subprocess.run(["nm", "-D", "--defined-only", lib.LIB_PATH], capture_output=True, text=True).stdout
+    exported = sorted(l.split()[-1] for l in out.splitlines() if " T " in l and l.split()[-1].startswith("omni_"))
+    assert exported == _declared()
+
+
+def test_argument_errors_need_no_gpu():
+    """Rejected arguments return before any HIP call, so these run on the CPU."""
+    lib = _lib().load()
+    p = ctypes.c_void_p(16)
+    assert lib.omni_router_select(p, p, p, p, 4, 8, 3, 0, None) == -4          # odd k
+    assert lib.omni_router_select(p, p, p, p, 4, 8, 66, 0, None) == -4         # k > r*r
+    assert lib.omni_router_select(p, p, p, p, 4, 8, 4, 7, None) == -3          # dtype
+    assert lib.omni_router_select(None, p, p, p, 4, 8, 4, 0, None) == -1       # NULL
+    assert lib.omni_router_select(None, None, None, None, 0, 8, 4, 0, None) == 0   # no tokens: nothing to do
+    assert lib.omni_expert_fwd(p, p, p, p, p, p, -1, 64, 16, 2, 0, 0, None, None) == -2
+    assert lib.omni_expert_fwd(p, p, p, p, p, p, 4, 64, 16, 2, 9, 0, None, None) == -3
+    assert lib.omni_schedule(p, p, p, p, 4, 2, 0, p, None) == -2
+    assert lib.omni_schedule(p, p, p, p, 4, 2, 16, None, None) == -6
+    assert lib.omni_mlp_fwd(p, p, p, p, None, p, 4, 64, 64, 2, p, None) == -5   # fp32 MLP not covered
+    assert lib.omni_schedule_workspace_bytes(4, 2, 100) >= 400
+
+
+def test_ops_fail_loudly_without_gpu():
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("GPU present")
+    from omni_moe.ops import hip
+    from omni_moe.ops.hip._lib import OmniHipError
+    z = torch.zeros(4, 8)
+    with pytest.raises(OmniHipError):
+        hip.hip_omni_router_func(z, z, 8, 4)
+    with pytest.raises(OmniHipError):
+        hip.hip_omni_expert_func(torch.zeros(4, 8), torch.zeros(16, 8), torch.zeros(16, 8), torch.zeros(4, 2), torch.zeros(4, 2, dtype=torch.int32))
+
+
+def test_reference_import_paths():
+    from omni_moe.modules.omni_moe import OmniMoE, OmniMoEConfig
+    from omni_moe.ops.triton import triton_omni_expert_func, triton_omni_mlp_func, triton_omni_router_func  # noqa: F401
+    layer = OmniMoE(OmniMoEConfig(64, 128, "silu", 256, 8))
+    assert sorted(layer.state_dict()) == sorted([
+        "gate_proj.weight", "up_proj.weight", "down_proj.weight", "router_gate_x.weight", "router_gate_y.weight",
+        "router_norm_x.running_mean", "router_norm_x.running_var", "router_norm_x.num_batches_tracked",
+        "router_norm_y.running_mean", "router_norm_y.running_var", "router_norm_y.num_batches_tracked",
+        "up_embed.weight", "down_embed.weight"])
+    assert layer.num_expert_sqrt == 16 and layer.up_embed.weight.shape == (256, 64)
+    with pytest.raises(ValueError):
+        OmniMoE(OmniMoEConfig(64, 128, "gelu", 256, 8))
