@@ -26,6 +26,9 @@ for p in (os.path.join(ROOT, "omni-moe_amd"), ROOT):
         sys.path.insert(0, p)
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+# Fabric-side bytes per launch (FETCH_SIZE + WRITE_SIZE, each scaled by a plain copy of known size) from the
+# rocprofv3 --pmc runs summarised in profiles/bench_layer_c4_hbm_counters.txt; counters cannot be read in-process.
+TRAFFIC_BYTES = {"expert_c3": 898.6e6, "expert_c4": 225.0e6, "gateup_c4": 134.6e6, "down_c4": 117.6e6}
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 
 
@@ -52,19 +55,19 @@ def time_call(torch, fn, reps, warmup=3):
     return sum(s.elapsed_time(e) for s, e in ev) / reps
 
 
-def hbm_entry(name, alg_bytes, ms, note=None):
+def hbm_entry(name, alg_bytes, ms, note=None, traffic=None):
     a = alg_bytes / (ms * 1e-3) / 1e9
     d = {"kernel": name, "bound": "hbm", "achieved": a, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": a / HBM_PEAK_GBS,
-         "traffic": None, "algorithmic_bytes": alg_bytes, "kernel_ms": ms}
+         "traffic": traffic, "algorithmic_bytes": alg_bytes, "kernel_ms": ms}
     if note:
         d["note"] = note
     return d
 
 
-def mfma_entry(name, flops, ms):
+def mfma_entry(name, flops, ms, traffic=None):
     a = flops / (ms * 1e-3) / 1e12
     return {"kernel": name, "bound": "mfma", "achieved": a, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-            "frac": a / MFMA_BF16_PEAK_TFLOPS, "traffic": None, "algorithmic_flops": flops, "kernel_ms": ms}
+            "frac": a / MFMA_BF16_PEAK_TFLOPS, "traffic": traffic, "algorithmic_flops": flops, "kernel_ms": ms}
 
 
 def main():
@@ -74,6 +77,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel passes (profiling runs)")
+    ap.add_argument("--calibration-copy", action="store_true",
+                    help="also run a plain 256 MiB device copy 3 times (known traffic, to scale HBM byte counters)")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU; --gpus must be 1 (no multi-GPU path exists)")
@@ -132,6 +137,14 @@ def main():
     torch.testing.assert_close(y_sub, want.float(), rtol=2e-2, atol=2e-2)
     layer.train()
 
+    if a.calibration_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
     if not a.no_kernels:
         reps = max(10, min(a.steps, 50))
         xf = dx.view(-1, H)
@@ -144,10 +157,10 @@ def main():
         ms_down = time_call(torch, lambda: hip.hip_linear_func(h, layer.down_proj.weight, e_out), reps)
         r = layer.num_expert_sqrt
         kernels = [
-            mfma_entry("gemm_nt_kernel<swiglu> (gate/up projection + SwiGLU), c4", 4 * T * H * I, ms_gateup),
-            mfma_entry("gemm_nt_kernel<residual> (down projection + experts add), c4", 2 * T * H * I, ms_down),
+            mfma_entry("gemm_nt_dma_kernel<swiglu> (gate/up projection + SwiGLU), c4", 4 * T * H * I, ms_gateup, TRAFFIC_BYTES["gateup_c4"]),
+            mfma_entry("gemm_nt_dma_kernel<residual> (down projection + experts add), c4", 2 * T * H * I, ms_down, TRAFFIC_BYTES["down_c4"]),
             hbm_entry("expert_gather_kernel, c4", expert_alg_bytes(T, H, k), ms_expert,
-                      "up/down tables (16 MiB) are cache-resident, so algorithmic bytes exceed HBM traffic"),
+                      "up/down tables (16 MiB) are cache-resident, so algorithmic bytes exceed HBM traffic", TRAFFIC_BYTES["expert_c4"]),
             {"kernel": "router stage (linear2 GEMM + BN partial + BN finalize + select), c4", "kernel_ms": ms_router,
              "algorithmic_flops": 4 * T * H * r},
         ]
@@ -157,7 +170,8 @@ def main():
         ms_e3 = time_call(torch, lambda: hip.hip_omni_expert_func(x3, up3, down3, g3, i3), reps)
         ms_s3 = time_call(torch, lambda: hip.hip_omni_schedule_func(i3, N), reps)
         kernels.append(hbm_entry("expert_gather_kernel, c3 (T=16384)", expert_alg_bytes(T3, H, k), ms_e3,
-                                 "up/down tables (16 MiB) are cache-resident, so algorithmic bytes exceed HBM traffic"))
+                                 "up/down tables (16 MiB) are cache-resident, so algorithmic bytes exceed HBM traffic",
+                                 TRAFFIC_BYTES["expert_c3"]))
         kernels.append(hbm_entry("schedule (fill+histogram+scan+scatter, 5 launches), c3", T3 * k * 14 + 8 * (N + 1), ms_s3))
         out["roofline"] = max(kernels[:3], key=lambda d: d["kernel_ms"])
         out["roofline_expert"] = kernels[-2]
