@@ -104,11 +104,11 @@ OMNI_API int32_t omni_expert_fwd(const void* x, const void* up_weight, const voi
  * kernel omni_mlp.py:102-177).  Two MFMA GEMMs: gate/up with the SwiGLU product formed in
  * the epilogue (gate and up are rounded to the storage dtype, the product is fp32, rounded
  * once, as omni_mlp.py:53-61), then the down projection.
- *   x [T,H]; gate_weight, up_weight [I,H]; down_weight [H,I]; y [T,H]  (dtype bf16 or f16)
+ *   x [T,H]; gate_weight, up_weight [I,H]; down_weight [H,I]; y [T,H]  (bf16, f16 or f32)
  *   residual : NULL, or [T,H] added to the rounded down projection and rounded again
  *              (the layer's final  mlp + experts , omni_moe.py:102)
  *   workspace: omni_mlp_workspace_bytes() bytes (the [T,I] SwiGLU activations)
- * H and I must be multiples of 8. */
+ * H and I must be multiples of 8 (of 4 for f32). */
 OMNI_API size_t omni_mlp_workspace_bytes(int64_t num_tokens, int32_t hidden_size, int32_t intermediate_size, int32_t dtype);
 OMNI_API int32_t omni_mlp_fwd(const void* x, const void* gate_weight, const void* up_weight, const void* down_weight,
                               const void* residual, void* y, int64_t num_tokens, int32_t hidden_size,
@@ -119,7 +119,7 @@ OMNI_API int32_t omni_mlp_fwd(const void* x, const void* gate_weight, const void
  * omni_linear_fwd:        y[T,out] = x[T,in] weight[out,in]^T [+ residual[T,out]]
  *                         (a bias-free nn.Linear / torch.matmul(., W.t()): interface.py:23-29,
  *                          omni_moe/modules/omni_moe.py:47-52,70-71)
- * in_features / hidden_size multiples of 8, out_features / intermediate_size of 4; bf16 or f16. */
+ * in_features / hidden_size multiples of 8 (4 for f32), out_features / intermediate_size of 4. */
 OMNI_API int32_t omni_swiglu_linear_fwd(const void* x, const void* gate_weight, const void* up_weight, void* h,
                                         int64_t num_tokens, int32_t hidden_size, int32_t intermediate_size,
                                         int32_t dtype, void* stream);
@@ -138,7 +138,7 @@ OMNI_API int32_t omni_linear2_fwd(const void* x, const void* weight_lo, const vo
  * Replaces omni_moe/modules/omni_moe.py:70-86 (two nn.Linear, two nn.BatchNorm1d, two
  * F.log_softmax, triton_omni_router_func, torch.exp).  Every stage rounds to the storage
  * dtype where the torch ops do.
- *   x [T,H]; weight_x, weight_y [r,H]                                     (dtype bf16 or f16)
+ *   x [T,H]; weight_x, weight_y [r,H]                                     (bf16, f16 or f32)
  *   running_mean_*, running_var_* [r] of dtype stats_dtype; num_batches_tracked_* int64
  *     scalars (may be NULL).  training != 0: batch statistics normalise (biased variance)
  *     and the buffers are UPDATED in place with `momentum` (unbiased variance), as

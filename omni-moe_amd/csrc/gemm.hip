@@ -33,26 +33,40 @@ constexpr int kGemmThreads = 256;
 
 enum : int { kEpiPlain = 0, kEpiSwiglu = 1, kEpiResidual = 2 };
 
+template <int DT> struct ElemBytes { static constexpr int value = (DT == kF32) ? 4 : 2; };
+
+// One 16-byte fragment per lane of each operand: 8 K-values per lane (32x32x16) for 16-bit
+// storage; for fp32 the 4 K-values per lane feed four 32x32x2 steps (lane halves pair up
+// k and k+4 -- any pairing works as long as both operands use the same one).
 template <int DT>
-__device__ __forceinline__ f32x16_t mfma32(const u32x4_t a, const u32x4_t b, const f32x16_t c) {
-  if constexpr (DT == kBF16)
+__device__ __forceinline__ f32x16_t mfma32(const u32x4_t a, const u32x4_t b, f32x16_t c) {
+  if constexpr (DT == kBF16) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
-  else
+  } else if constexpr (DT == kF16) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const uint32_t ae = a[e], be = b[e];
+      c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(ae), __uint_as_float(be), c, 0, 0, 0);
+    }
+    return c;
+  }
 }
 
 template <int DT>
 __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
   if constexpr (DT == kBF16) return pack_bf16(lo, hi);
-  else return pack_f16(lo, hi);
+  else if constexpr (DT == kF16) return pack_f16(lo, hi);
+  else return 0u;
 }
 
-struct GemmArgs {
-  const uint16_t* a;      // [M, K]  activations
-  const uint16_t* b0;     // [N, K]  weights (gate weights for SwiGLU)
-  const uint16_t* b1;     // [N, K]  up weights (SwiGLU only)
-  const uint16_t* res;    // [M, N]  added to the result (residual epilogue only)
-  uint16_t* c;            // [M, N]
+struct GemmArgs {           // all element offsets below are scaled by the element size of DT
+  const uint8_t* a;       // [M, K]  activations
+  const uint8_t* b0;      // [N, K]  weights (gate weights for SwiGLU)
+  const uint8_t* b1;      // [N, K]  up weights (SwiGLU), or the upper half of the columns (plain)
+  const uint8_t* res;     // [M, N]  added to the result (residual epilogue only)
+  uint8_t* c;             // [M, N]
   int M, N, K;            // N = output columns
   int tiles_m, tiles_n;
   int patch_m, patch_n;   // XCD patch shape (0 = plain order)
@@ -134,33 +148,44 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, f32x16_t (&acc)
             // silu(gate)*up in fp32 and rounds once (omni_mlp.py:53-61)
             const float gt = Elem<DT>::round(acc[i][j][q4 * 4 + q]);
             const float up = Elem<DT>::round(acc[i][j + TNO][q4 * 4 + q]);
-            v[q] = silu_fast(gt) * up;
+            v[q] = (DT == kF32) ? silu_f32(gt) * up : silu_fast(gt) * up;
           } else {
             v[q] = acc[i][j][q4 * 4 + q];
           }
         }
-        const int64_t o = (int64_t)m * g.N + n;
+        const int64_t o = ((int64_t)m * g.N + n) * ElemBytes<DT>::value;
         if constexpr (EPI == kEpiResidual) {
           // y = round(h Wd^T) + e, rounded again: the reference adds two stored tensors
-          const u32x2_t r = *(const u32x2_t*)(g.res + o);
-          const uint32_t r0 = r[0], r1 = r[1];
-          if constexpr (DT == kBF16) {
-            v[0] = Elem<DT>::round(v[0]) + bf16_lo(r0); v[1] = Elem<DT>::round(v[1]) + bf16_hi(r0);
-            v[2] = Elem<DT>::round(v[2]) + bf16_lo(r1); v[3] = Elem<DT>::round(v[3]) + bf16_hi(r1);
+          if constexpr (DT == kF32) {
+            const f32x4_t r = *(const f32x4_t*)(g.res + o);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) v[q] += r[q];
           } else {
-            v[0] = Elem<DT>::round(v[0]) + f16_bits_to_f32(r0 & 0xffff); v[1] = Elem<DT>::round(v[1]) + f16_bits_to_f32(r0 >> 16);
-            v[2] = Elem<DT>::round(v[2]) + f16_bits_to_f32(r1 & 0xffff); v[3] = Elem<DT>::round(v[3]) + f16_bits_to_f32(r1 >> 16);
+            const u32x2_t r = *(const u32x2_t*)(g.res + o);
+            const uint32_t r0 = r[0], r1 = r[1];
+            if constexpr (DT == kBF16) {
+              v[0] = Elem<DT>::round(v[0]) + bf16_lo(r0); v[1] = Elem<DT>::round(v[1]) + bf16_hi(r0);
+              v[2] = Elem<DT>::round(v[2]) + bf16_lo(r1); v[3] = Elem<DT>::round(v[3]) + bf16_hi(r1);
+            } else {
+              v[0] = Elem<DT>::round(v[0]) + f16_bits_to_f32(r0 & 0xffff); v[1] = Elem<DT>::round(v[1]) + f16_bits_to_f32(r0 >> 16);
+              v[2] = Elem<DT>::round(v[2]) + f16_bits_to_f32(r1 & 0xffff); v[3] = Elem<DT>::round(v[3]) + f16_bits_to_f32(r1 >> 16);
+            }
           }
         }
-        u32x2_t w = {pack2<DT>(v[0], v[1]), pack2<DT>(v[2], v[3])};
-        *(u32x2_t*)(g.c + o) = w;
+        if constexpr (DT == kF32) {
+          *(f32x4_t*)(g.c + o) = f32x4_t{v[0], v[1], v[2], v[3]};
+        } else {
+          u32x2_t w = {pack2<DT>(v[0], v[1]), pack2<DT>(v[2], v[3])};
+          *(u32x2_t*)(g.c + o) = w;
+        }
       }
     }
   }
 }
 
-// 16-bit storage, TM x TN MFMA tiles per wave.  For the SwiGLU epilogue the first TN/2
-// tiles of a wave are gate columns and the last TN/2 the matching up columns.
+// Register-staged kernel, any storage dtype: TM x TN MFMA tiles per wave, K advances by one
+// 128-byte row (64 16-bit or 32 fp32 values).  For the SwiGLU epilogue the first TN/2 tiles of
+// a wave are gate columns and the last TN/2 the matching up columns.
 template <int DT, int TM, int TN, int EPI>
 __global__ __launch_bounds__(kGemmThreads, 1) void gemm_nt_kernel(const GemmArgs g) {
   constexpr int BM = 2 * TM * 32;                 // rows of A per block
@@ -178,21 +203,22 @@ __global__ __launch_bounds__(kGemmThreads, 1) void gemm_nt_kernel(const GemmArgs
   const int m0 = tile_m * BM, n0 = tile_n * BN;
 
   // ---- global -> register staging: thread owns 16-byte chunk (tid%8) of rows tid/8 + 32*p
+  constexpr int ES = ElemBytes<DT>::value, CE = 16 / ES, BKE = 128 / ES;   // chunk / tile width in elements
   const int ld_chunk = tid & 7, ld_row = tid >> 3;
   constexpr int PA = BM / 32, PB = BR / 32;
-  const uint16_t* a_ptr[PA];
-  const uint16_t* b_ptr[PB];
+  const uint8_t* a_ptr[PA];
+  const uint8_t* b_ptr[PB];
 #pragma unroll
   for (int p = 0; p < PA; ++p) {
     int row = m0 + p * 32 + ld_row;
     row = row < g.M ? row : g.M - 1;                     // clamp: tail rows are never stored
-    a_ptr[p] = g.a + (int64_t)row * g.K + ld_chunk * 8;
+    a_ptr[p] = g.a + ((int64_t)row * g.K + ld_chunk * CE) * ES;
   }
 #pragma unroll
   for (int p = 0; p < PB; ++p) {
     // LDS weight row p*32+ld_row belongs to wave column p/TN, tile p%TN
     const int pw = p / TN, pj = p % TN;
-    const uint16_t* base = g.b0;
+    const uint8_t* base = g.b0;
     int col;
     if constexpr (EPI == kEpiSwiglu) {
       base = (pj < TNO) ? g.b0 : g.b1;
@@ -205,17 +231,17 @@ __global__ __launch_bounds__(kGemmThreads, 1) void gemm_nt_kernel(const GemmArgs
       // optional second weight matrix supplies the upper half of the output columns
       if (g.b1 && col >= g.N / 2) { base = g.b1; col -= g.N / 2; }
     }
-    b_ptr[p] = base + (int64_t)col * g.K + ld_chunk * 8;
+    b_ptr[p] = base + ((int64_t)col * g.K + ld_chunk * CE) * ES;
   }
   const int lds_wr = ld_row * kRowBytes + ld_chunk * 16;
 
   u32x4_t ra[PA], rb[PB];
   auto load_tile = [&](int k0) {
-    const bool ok = k0 + ld_chunk * 8 < g.K;             // K is a multiple of 8: whole chunks
+    const bool ok = k0 + ld_chunk * CE < g.K;            // K is a multiple of the chunk: whole chunks
 #pragma unroll
-    for (int p = 0; p < PA; ++p) ra[p] = ok ? *(const u32x4_t*)(a_ptr[p] + k0) : u32x4_t{0, 0, 0, 0};
+    for (int p = 0; p < PA; ++p) ra[p] = ok ? *(const u32x4_t*)(a_ptr[p] + (int64_t)k0 * ES) : u32x4_t{0, 0, 0, 0};
 #pragma unroll
-    for (int p = 0; p < PB; ++p) rb[p] = ok ? *(const u32x4_t*)(b_ptr[p] + k0) : u32x4_t{0, 0, 0, 0};
+    for (int p = 0; p < PB; ++p) rb[p] = ok ? *(const u32x4_t*)(b_ptr[p] + (int64_t)k0 * ES) : u32x4_t{0, 0, 0, 0};
   };
   auto store_tile = [&](int stage) {
     uint8_t* sa = lds + stage * kStageBytes;
@@ -234,20 +260,20 @@ __global__ __launch_bounds__(kGemmThreads, 1) void gemm_nt_kernel(const GemmArgs
 #pragma unroll
       for (int q = 0; q < 16; ++q) acc[i][j][q] = 0.f;
 
-  // fragment read offsets: lane reads row (lane%32), 16-byte chunk (lane/32) of a K=16 slab
+  // fragment read offsets: lane reads row (lane%32), 16-byte chunk (lane/32) of a 32-byte slab
   const int frag_off = (lane & 31) * kRowBytes + (lane >> 5) * 16;
   const int a_frag = (wm * TM * 32) * kRowBytes + frag_off;
   const int b_frag = BM * kRowBytes + (wn * TN * 32) * kRowBytes + frag_off;
 
-  const int num_kt = (g.K + kBK - 1) / kBK;
+  const int num_kt = (g.K + BKE - 1) / BKE;
   load_tile(0);
   store_tile(0);
   __syncthreads();
   for (int kt = 0; kt < num_kt; ++kt) {
     const uint8_t* st = lds + (kt & 1) * kStageBytes;
-    if (kt + 1 < num_kt) load_tile((kt + 1) * kBK);
+    if (kt + 1 < num_kt) load_tile((kt + 1) * BKE);
 #pragma unroll
-    for (int slab = 0; slab < kBK / 16; ++slab) {
+    for (int slab = 0; slab < 4; ++slab) {
       u32x4_t af[TM], bf[TN];
 #pragma unroll
       for (int i = 0; i < TM; ++i) af[i] = *(const u32x4_t*)(st + a_frag + i * 32 * kRowBytes + slab * 32);
@@ -315,13 +341,13 @@ __global__ __launch_bounds__(kGemmThreads, 1) void gemm_nt_dma_kernel(const Gemm
     const int c = swizzle<BK>(rl, lane % kCpr);        // an involution: position -> logical chunk
     int row = m0 + rl;
     row = row < g.M ? row : g.M - 1;                    // clamp: tail rows are never stored
-    a_src[p] = (const uint8_t*)(g.a + (int64_t)row * g.K + c * 8);
+    a_src[p] = g.a + ((int64_t)row * g.K + c * 8) * 2;
   }
 #pragma unroll
   for (int p = 0; p < PB; ++p) {
     const int rl = (4 * p + wave) * kRpi + lane / kCpr;   // row of the weight tile in LDS
     const int c = swizzle<BK>(rl, lane % kCpr);
-    const uint16_t* base = g.b0;
+    const uint8_t* base = g.b0;
     int col;
     if constexpr (EPI == kEpiSwiglu) {
       const int pw = rl / (TN * 32), pj = (rl >> 5) % TN;
@@ -334,7 +360,7 @@ __global__ __launch_bounds__(kGemmThreads, 1) void gemm_nt_dma_kernel(const Gemm
     if constexpr (EPI == kEpiPlain) {
       if (g.b1 && col >= g.N / 2) { base = g.b1; col -= g.N / 2; }
     }
-    b_src[p] = (const uint8_t*)(base + (int64_t)col * g.K + c * 8);
+    b_src[p] = base + ((int64_t)col * g.K + c * 8) * 2;
   }
 
   auto issue_tile = [&](int kt) {
@@ -452,7 +478,7 @@ static hipError_t launch_gemm(GemmArgs g, hipStream_t s) {
   constexpr int kDmaBK = 64;
   constexpr int kFit = (160 * 1024) / ((BM + BR) * kDmaBK * 2);
   constexpr int kDmaStages = kFit > 4 ? 4 : kFit;
-  if (g.K % kDmaBK == 0) {
+  if constexpr (DT != kF32) if (g.K % kDmaBK == 0) {
     constexpr int kDmaLds = kDmaStages * (BM + BR) * kDmaBK * 2;
     static_assert(kDmaLds <= 160 * 1024, "LDS ring exceeds 160 KiB");
     auto kern = gemm_nt_dma_kernel<DT, TM, TN, EPI, kDmaBK, kDmaStages>;
@@ -476,10 +502,10 @@ static hipError_t launch_gemm(GemmArgs g, hipStream_t s) {
   return hipGetLastError();
 }
 
-// Shape rules shared by the entry points: K a multiple of 8 (16-byte chunks), N of 4.
-static int check_gemm(int64_t M, int64_t N, int64_t K) {
+// Shape rules shared by the entry points: K a multiple of a 16-byte chunk, N of 4.
+static int check_gemm(int64_t M, int64_t N, int64_t K, int elem_bytes) {
   if (M < 0 || N <= 0 || K <= 0 || M > INT32_MAX / 2 || N > INT32_MAX / 2 || K > INT32_MAX / 2) return OMNI_ERR_SHAPE;
-  if (K % 8 != 0 || N % 4 != 0) return OMNI_ERR_SHAPE;
+  if (K % (16 / elem_bytes) != 0 || N % 4 != 0) return OMNI_ERR_SHAPE;
   return OMNI_OK;
 }
 
@@ -489,9 +515,9 @@ static int to_code(hipError_t e) { return e == hipSuccess ? OMNI_OK : OMNI_ERR_H
 template <int DT>
 static int gemm_plain(const void* a, const void* b, const void* b_hi, const void* res, void* c, int64_t M, int64_t N, int64_t K, hipStream_t s,
                       float* part_mean = nullptr, float* part_m2 = nullptr) {
-  if (int e = check_gemm(M, N, K)) return e;
+  if (int e = check_gemm(M, N, K, ElemBytes<DT>::value)) return e;
   if (M == 0) return OMNI_OK;
-  GemmArgs g{(const uint16_t*)a, (const uint16_t*)b, (const uint16_t*)b_hi, (const uint16_t*)res, (uint16_t*)c, (int)M, (int)N, (int)K, 0, 0, 0, 0, nullptr, nullptr};
+  GemmArgs g{(const uint8_t*)a, (const uint8_t*)b, (const uint8_t*)b_hi, (const uint8_t*)res, (uint8_t*)c, (int)M, (int)N, (int)K, 0, 0, 0, 0, nullptr, nullptr};
   g.part_mean = part_mean;
   g.part_m2 = part_m2;
   const int64_t big = ((M + 255) / 256) * ((N + 255) / 256), mid = ((M + 127) / 128) * ((N + 127) / 128);
@@ -510,9 +536,9 @@ static int gemm_plain(const void* a, const void* b, const void* b_hi, const void
 
 template <int DT>
 static int gemm_swiglu(const void* x, const void* wg, const void* wu, void* h, int64_t M, int64_t I, int64_t K, hipStream_t s) {
-  if (int e = check_gemm(M, I, K)) return e;
+  if (int e = check_gemm(M, I, K, ElemBytes<DT>::value)) return e;
   if (M == 0) return OMNI_OK;
-  GemmArgs g{(const uint16_t*)x, (const uint16_t*)wg, (const uint16_t*)wu, nullptr, (uint16_t*)h, (int)M, (int)I, (int)K, 0, 0, 0, 0, nullptr, nullptr};
+  GemmArgs g{(const uint8_t*)x, (const uint8_t*)wg, (const uint8_t*)wu, nullptr, (uint8_t*)h, (int)M, (int)I, (int)K, 0, 0, 0, 0, nullptr, nullptr};
   const int64_t big = ((M + 255) / 256) * ((I + 127) / 128);
   hipError_t err;
   if (big >= 200) err = launch_gemm<DT, 4, 4, kEpiSwiglu>(g, s);
@@ -528,7 +554,8 @@ int omni_gemm_router_projection(const void* x, const void* wx, const void* wy, v
   hipStream_t s = (hipStream_t)stream;
   if (dtype == OMNI_BF16) return gemm_plain<kBF16>(x, wx, wy, nullptr, z, T, 2 * (int64_t)r, H, s, part_mean, part_m2);
   if (dtype == OMNI_F16) return gemm_plain<kF16>(x, wx, wy, nullptr, z, T, 2 * (int64_t)r, H, s, part_mean, part_m2);
-  return OMNI_ERR_UNSUPPORTED;
+  if (dtype == OMNI_F32) return gemm_plain<kF32>(x, wx, wy, nullptr, z, T, 2 * (int64_t)r, H, s, part_mean, part_m2);
+  return OMNI_ERR_DTYPE;
 }
 
 extern "C" OMNI_API size_t omni_mlp_workspace_bytes(int64_t num_tokens, int32_t hidden_size, int32_t intermediate_size, int32_t dtype) {
@@ -555,7 +582,9 @@ extern "C" OMNI_API int32_t omni_mlp_fwd(const void* x, const void* gate_weight,
     case OMNI_F16:
       if ((e = gemm_swiglu<kF16>(x, gate_weight, up_weight, workspace, num_tokens, intermediate_size, hidden_size, s))) return e;
       return gemm_plain<kF16>(workspace, down_weight, nullptr, residual, y, num_tokens, hidden_size, intermediate_size, s);
-    case OMNI_F32: return OMNI_ERR_UNSUPPORTED;
+    case OMNI_F32:
+      if ((e = gemm_swiglu<kF32>(x, gate_weight, up_weight, workspace, num_tokens, intermediate_size, hidden_size, s))) return e;
+      return gemm_plain<kF32>(workspace, down_weight, nullptr, residual, y, num_tokens, hidden_size, intermediate_size, s);
     default: return OMNI_ERR_DTYPE;
   }
 }
@@ -570,7 +599,7 @@ extern "C" OMNI_API int32_t omni_swiglu_linear_fwd(const void* x, const void* ga
   switch (dtype) {
     case OMNI_BF16: return gemm_swiglu<kBF16>(x, gate_weight, up_weight, h, num_tokens, intermediate_size, hidden_size, s);
     case OMNI_F16: return gemm_swiglu<kF16>(x, gate_weight, up_weight, h, num_tokens, intermediate_size, hidden_size, s);
-    case OMNI_F32: return OMNI_ERR_UNSUPPORTED;
+    case OMNI_F32: return gemm_swiglu<kF32>(x, gate_weight, up_weight, h, num_tokens, intermediate_size, hidden_size, s);
     default: return OMNI_ERR_DTYPE;
   }
 }
@@ -584,7 +613,7 @@ extern "C" OMNI_API int32_t omni_linear_fwd(const void* x, const void* weight, c
   switch (dtype) {
     case OMNI_BF16: return gemm_plain<kBF16>(x, weight, nullptr, residual, y, num_tokens, out_features, in_features, s);
     case OMNI_F16: return gemm_plain<kF16>(x, weight, nullptr, residual, y, num_tokens, out_features, in_features, s);
-    case OMNI_F32: return OMNI_ERR_UNSUPPORTED;
+    case OMNI_F32: return gemm_plain<kF32>(x, weight, nullptr, residual, y, num_tokens, out_features, in_features, s);
     default: return OMNI_ERR_DTYPE;
   }
 }
@@ -600,7 +629,7 @@ extern "C" OMNI_API int32_t omni_linear2_fwd(const void* x, const void* weight_l
   switch (dtype) {
     case OMNI_BF16: return gemm_plain<kBF16>(x, weight_lo, weight_hi, nullptr, y, num_tokens, n, in_features, s);
     case OMNI_F16: return gemm_plain<kF16>(x, weight_lo, weight_hi, nullptr, y, num_tokens, n, in_features, s);
-    case OMNI_F32: return OMNI_ERR_UNSUPPORTED;
+    case OMNI_F32: return gemm_plain<kF32>(x, weight_lo, weight_hi, nullptr, y, num_tokens, n, in_features, s);
     default: return OMNI_ERR_DTYPE;
   }
 }

@@ -390,7 +390,7 @@ extern "C" OMNI_API int32_t omni_router_fwd(const void* x, const void* weight_x,
   const int r = num_expert_sqrt, k = num_experts_per_token;
   if (num_tokens < 0 || num_tokens > INT32_MAX / 256 || r <= 0 || hidden_size <= 0) return OMNI_ERR_SHAPE;
   if (k < 0 || (int64_t)k > (int64_t)r * r || k > 128 || (k & 1)) return OMNI_ERR_TOPK;
-  if (dtype != OMNI_BF16 && dtype != OMNI_F16) return dtype == OMNI_F32 ? OMNI_ERR_UNSUPPORTED : OMNI_ERR_DTYPE;
+  if (dtype != OMNI_BF16 && dtype != OMNI_F16 && dtype != OMNI_F32) return OMNI_ERR_DTYPE;
   if (stats_dtype != OMNI_BF16 && stats_dtype != OMNI_F16 && stats_dtype != OMNI_F32) return OMNI_ERR_DTYPE;
   if (num_tokens == 0) return OMNI_OK;
   if (!x || !weight_x || !weight_y || !running_mean_x || !running_var_x || !running_mean_y || !running_var_y) return OMNI_ERR_NULL;
@@ -399,7 +399,8 @@ extern "C" OMNI_API int32_t omni_router_fwd(const void* x, const void* weight_x,
   hipStream_t s = (hipStream_t)stream;
   const size_t strips = ((size_t)num_tokens + kBnRows - 1) / kBnRows;
   char* w = (char*)workspace;
-  void* z = w;                       w += align256((size_t)num_tokens * 2 * r * 2);
+  const size_t es = dtype == OMNI_F32 ? 4 : 2;
+  void* z = w;                       w += align256((size_t)num_tokens * 2 * r * es);
   float* stats = (float*)w;          w += align256((size_t)4 * r * 4);
   float* part_mean = (float*)w;      w += align256(strips * 2 * r * 4);
   float* part_m2 = (float*)w;
@@ -415,7 +416,6 @@ extern "C" OMNI_API int32_t omni_router_fwd(const void* x, const void* weight_x,
   hipError_t err = hipGetLastError();
   if (err != hipSuccess) return OMNI_ERR_HIP_BASE + (int)err;
   if (k == 0) return OMNI_OK;
-  const size_t es = 2;
   SelectArgs g{z, (const char*)z + (size_t)r * es, 2 * r, stats, scores, gates, indices, (int)num_tokens, r, k, 0, dtype};
   return select_dispatch(g, s);
 }

@@ -147,8 +147,8 @@ def hip_omni_mlp_func(
     I = gate_weight.size(0)
     if gate_weight.shape != (I, H) or up_weight.shape != (I, H) or down_weight.shape != (H, I):
         raise ValueError("expected gate/up weights (intermediate, hidden) and down weight (hidden, intermediate)")
-    if x.dtype not in (torch.bfloat16, torch.float16) or any(t.dtype != x.dtype for t in (gate_weight, up_weight, down_weight)):
-        raise TypeError("x and the weights must share a dtype in {bfloat16, float16}")
+    if x.dtype not in _lib.DTYPE_CODE or any(t.dtype != x.dtype for t in (gate_weight, up_weight, down_weight)):
+        raise TypeError("x and the weights must share a dtype in {bfloat16, float16, float32}")
     tensors = [x, gate_weight, up_weight, down_weight]
     if residual is not None:
         if residual.shape != x.shape or residual.dtype != x.dtype:
@@ -172,8 +172,8 @@ def hip_linear_func(x: torch.Tensor, weight: torch.Tensor, residual: Optional[to
     """x @ weight.T (+ residual) for a bias-free ``nn.Linear`` (reference omni_moe.py:70-71, interface.py:23-29)."""
     if x.dim() != 2 or weight.dim() != 2 or weight.size(1) != x.size(1):
         raise ValueError("expected x (tokens, in) and weight (out, in)")
-    if x.dtype not in (torch.bfloat16, torch.float16) or weight.dtype != x.dtype:
-        raise TypeError("x and weight must share a dtype in {bfloat16, float16}")
+    if x.dtype not in _lib.DTYPE_CODE or weight.dtype != x.dtype:
+        raise TypeError("x and weight must share a dtype in {bfloat16, float16, float32}")
     if residual is not None and (residual.shape != (x.size(0), weight.size(0)) or residual.dtype != x.dtype):
         raise ValueError("residual must be (tokens, out) in x's dtype")
     dev = _lib.require_gpu(x, weight)
@@ -191,8 +191,8 @@ def hip_swiglu_linear_func(x: torch.Tensor, gate_weight: torch.Tensor, up_weight
     """silu(x gate^T) * (x up^T): the first half of the MLP op as one GEMM with a fused epilogue."""
     if x.dim() != 2 or gate_weight.shape != up_weight.shape or gate_weight.dim() != 2 or gate_weight.size(1) != x.size(1):
         raise ValueError("expected x (tokens, hidden) and gate/up weights (intermediate, hidden)")
-    if x.dtype not in (torch.bfloat16, torch.float16) or gate_weight.dtype != x.dtype or up_weight.dtype != x.dtype:
-        raise TypeError("x and the weights must share a dtype in {bfloat16, float16}")
+    if x.dtype not in _lib.DTYPE_CODE or gate_weight.dtype != x.dtype or up_weight.dtype != x.dtype:
+        raise TypeError("x and the weights must share a dtype in {bfloat16, float16, float32}")
     dev = _lib.require_gpu(x, gate_weight, up_weight)
     x, gate_weight, up_weight = map(_c, (x, gate_weight, up_weight))
     h = torch.empty((x.size(0), gate_weight.size(0)), device=dev, dtype=x.dtype)
@@ -228,8 +228,8 @@ def hip_omni_router_fwd_func(
     """
     if x.dim() != 2 or weight_x.shape != weight_y.shape or weight_x.dim() != 2 or weight_x.size(1) != x.size(1):
         raise ValueError("expected x (tokens, hidden) and two router weights (num_expert_sqrt, hidden)")
-    if x.dtype not in (torch.bfloat16, torch.float16) or weight_x.dtype != x.dtype or weight_y.dtype != x.dtype:
-        raise TypeError("x and the router weights must share a dtype in {bfloat16, float16}")
+    if x.dtype not in _lib.DTYPE_CODE or weight_x.dtype != x.dtype or weight_y.dtype != x.dtype:
+        raise TypeError("x and the router weights must share a dtype in {bfloat16, float16, float32}")
     stats = (running_mean_x, running_var_x, running_mean_y, running_var_y)
     r, k = weight_x.size(0), int(num_experts_per_token)
     if any(t.dtype != running_mean_x.dtype or t.shape != (r,) or not t.is_contiguous() for t in stats):

@@ -70,7 +70,8 @@ def test_argument_errors_need_no_gpu():
     assert lib.omni_expert_fwd(p, p, p, p, p, p, 4, 64, 16, 2, 9, 0, None, None) == -3
     assert lib.omni_schedule(p, p, p, p, 4, 2, 0, p, None) == -2
     assert lib.omni_schedule(p, p, p, p, 4, 2, 16, None, None) == -6
-    assert lib.omni_mlp_fwd(p, p, p, p, None, p, 4, 64, 64, 2, p, None) == -5   # fp32 MLP not covered
+    assert lib.omni_mlp_fwd(p, p, p, p, None, p, 4, 64, 62, 0, p, None) == -2   # intermediate size not a multiple of 8
+    assert lib.omni_mlp_fwd(p, p, p, p, None, p, 4, 64, 64, 0, None, None) == -6 # no workspace
     assert lib.omni_schedule_workspace_bytes(4, 2, 100) >= 400
 
 

@@ -41,6 +41,22 @@ def test_mlp_matches_oracle(case, dtype, device):
     torch.testing.assert_close(got_r, want_r.to(dtype).float(), rtol=1e-2, atol=1e-2 * max(scale, 1.0))
 
 
+@pytest.mark.parametrize("case", [(512, 256, 1024), (300, 100, 260), (64, 1024, 512)], ids=lambda c: f"T{c[0]}-H{c[1]}-I{c[2]}")
+def test_mlp_fp32_matches_oracle(case, device):
+    T, H, I = case
+    g = torch.Generator().manual_seed(7)
+    x = torch.randn(T, H, generator=g)
+    wg, wu, wd = torch.randn(I, H, generator=g) * 0.05, torch.randn(I, H, generator=g) * 0.05, torch.randn(H, I, generator=g) * 0.05
+    res = torch.randn(T, H, generator=g)
+    print(f"mlp fp32 T={T} H={H} I={I}", flush=True)
+    want = oracle.mlp_forward(x.double(), wg.double(), wu.double(), wd.double()).float()
+    d = [t.to(device) for t in (x, wg, wu, wd)]
+    got = _ops().hip_omni_mlp_func(*d).cpu()
+    torch.testing.assert_close(got, want, rtol=1e-4, atol=1e-5 * max(1.0, want.abs().max().item()))
+    got_r = _ops().hip_omni_mlp_func(*d, residual=res.to(device)).cpu()
+    torch.testing.assert_close(got_r, want + res, rtol=1e-4, atol=1e-5 * max(1.0, want.abs().max().item()))
+
+
 ROUTER_FWD_CASES = [(4096, 1024, 64, 16), (1024, 256, 32, 8), (2048, 2048, 512, 32), (300, 520, 36, 10)]
 
 
@@ -152,3 +168,93 @@ def test_layer_matches_oracle(case, training, device):
         set_agree = (got_i.cpu().sort(-1).values == want_i.sort(-1).values).float().mean().item()
         print(f"   expert-set agreement {set_agree:.5f}")
         assert set_agree >= 0.999
+
+
+@pytest.mark.parametrize("training", [True, False], ids=["train", "eval"])
+def test_layer_config1_fp32(training, device):
+    """BASELINE config 1, the reference's CPU-runnable case, at full size in fp32:
+    1 x 512 tokens, hidden 256, intermediate 1024, 1024 experts (32 x 32), top-8, seed 0."""
+    from omni_moe.modules.omni_moe import OmniMoE, OmniMoEConfig
+    T, H, I, N, k = 512, 256, 1024, 1024, 8
+    x, w = oracle.make_layer_inputs(0, T, H, I, N, dtype=torch.float32)
+    layer = OmniMoE(OmniMoEConfig(H, I, "silu", N, k))
+    layer.load_state_dict({"gate_proj.weight": w.gate_proj, "up_proj.weight": w.up_proj, "down_proj.weight": w.down_proj,
+                           "router_gate_x.weight": w.router_gate_x, "router_gate_y.weight": w.router_gate_y,
+                           "up_embed.weight": w.up_embed, "down_embed.weight": w.down_embed}, strict=False)
+    layer = layer.to(device).train(training)
+    bx, by = oracle.BNState.fresh(32), oracle.BNState.fresh(32)
+    print(f"layer config 1 fp32 training={training}", flush=True)
+    want, want_g, want_i = oracle.moe_forward(x, w, bx, by, k, training)
+    got = layer(x.to(device))
+    torch.cuda.synchronize()
+    assert got.dtype == torch.float32
+    layer.eval()
+    if training:   # route again with the updated buffers on both sides
+        want_g, want_i, _ = oracle.router_forward(x.view(-1, H), w.router_gate_x, w.router_gate_y, bx, by, k, False)
+    got_g, got_i = layer.route(x.view(-1, H).to(device))
+    # fp32 scores: ties practically never occur, so the ids are forced up to fp32 summation order
+    set_agree = (got_i.cpu().sort(-1).values == want_i.sort(-1).values).all(-1).float().mean().item()
+    print(f"   tokens with identical expert sets: {set_agree:.5f}")
+    assert set_agree >= 0.999
+    torch.testing.assert_close(got_g.cpu(), want_g, rtol=1e-3, atol=1e-6)
+    same = (got_i.cpu().sort(-1).values == want_i.sort(-1).values).all(-1) if not training else torch.ones(T, dtype=torch.bool)
+    torch.testing.assert_close(got.cpu().view(-1, H)[same], want.view(-1, H)[same], rtol=1e-3, atol=2e-5)
+    if training:
+        torch.testing.assert_close(layer.router_norm_x.running_mean.cpu(), bx.running_mean, rtol=1e-4, atol=1e-6)
+        torch.testing.assert_close(layer.router_norm_y.running_var.cpu(), by.running_var, rtol=1e-4, atol=1e-6)
+
+
+def test_layer_config5_large_skewed(device):
+    """BASELINE config 5: 8 x 4096 tokens, hidden 2048, intermediate 8192, 262144 experts
+    (512 x 512 keys), top-32, bf16, router key popularity ~ Zipf(1.1), seed 4.
+
+    The reference's router has no bias (omni_moe.py:47-52), so the per-key bias b_i = -1.1*ln(1+i)
+    enters through eval-mode BatchNorm buffers: running_mean = -b, running_var = 1 - eps.  The whole
+    batch runs on the GPU; the oracle checks a token subset (eval mode is token-independent) and the
+    schedule of all 1M pairs."""
+    from omni_moe.modules.omni_moe import OmniMoE, OmniMoEConfig
+    T, H, I, N, k, r = 32768, 2048, 8192, 262144, 32, 512
+    g = torch.Generator().manual_seed(4)
+    n = lambda *s, std=1.0: (torch.randn(*s, generator=g) * std).bfloat16()
+    x = n(8, 4096, H)
+    w = oracle.MoEWeights(gate_proj=n(I, H, std=0.02), up_proj=n(I, H, std=0.02), down_proj=n(H, I, std=0.02),
+                          router_gate_x=n(r, H, std=0.02), router_gate_y=n(r, H, std=0.02),
+                          up_embed=n(N, H, std=0.02), down_embed=n(N, H, std=0.02))
+    bias = -1.1 * torch.log1p(torch.arange(r, dtype=torch.float32))
+    layer = OmniMoE(OmniMoEConfig(H, I, "silu", N, k))
+    layer.load_state_dict({"gate_proj.weight": w.gate_proj, "up_proj.weight": w.up_proj, "down_proj.weight": w.down_proj,
+                           "router_gate_x.weight": w.router_gate_x, "router_gate_y.weight": w.router_gate_y,
+                           "up_embed.weight": w.up_embed, "down_embed.weight": w.down_embed}, strict=False)
+    for bn in (layer.router_norm_x, layer.router_norm_y):
+        bn.running_mean.copy_(-bias)
+        bn.running_var.fill_(1.0 - bn.eps)
+    layer = layer.to(device=device, dtype=torch.bfloat16).eval()
+    print("layer config 5: 32768 tokens, 262144 experts, top-32", flush=True)
+    y = layer(x.to(device))
+    gates, ids = layer.route(x.view(-1, H).to(device))
+    torch.cuda.synchronize()
+    assert y.shape == x.shape and torch.isfinite(y.float()).all()
+    # schedule of the real, skewed assignment: offsets exact, pairs a grouped permutation
+    sched = _ops().hip_omni_schedule_func(ids, N)
+    ids_c = ids.cpu()
+    want_off, want_pairs, _ = oracle.schedule(ids_c, N)
+    assert torch.equal(sched.offsets.cpu(), want_off)
+    flat = ids_c.reshape(-1).long()
+    pairs = sched.sorted_pair_ids.cpu().long()
+    assert torch.equal(flat[pairs], flat[want_pairs.long()])
+    assert torch.equal(torch.sort(pairs).values, torch.arange(T * k))
+    seg = (want_off[1:] - want_off[:-1]).float()
+    print(f"   pairs per expert: max {int(seg.max())}, mean over used {seg[seg > 0].mean():.1f}, used experts {int((seg > 0).sum())}")
+    assert seg.max() > 100 * seg[seg > 0].mean()          # the skew is there
+    # oracle on a token subset (buffers as the bf16 module holds them)
+    sub = torch.arange(0, T, 128)
+    bx = oracle.BNState(layer.router_norm_x.running_mean.float().cpu(), layer.router_norm_x.running_var.float().cpu(), torch.zeros((), dtype=torch.long))
+    by = oracle.BNState(layer.router_norm_y.running_mean.float().cpu(), layer.router_norm_y.running_var.float().cpu(), torch.zeros((), dtype=torch.long))
+    xs = x.view(-1, H)[sub].unsqueeze(0)
+    want, want_g, want_i = oracle.moe_forward(xs, w, bx, by, k, training=False)
+    got_i = ids_c[sub]
+    set_agree = (got_i.sort(-1).values == want_i.sort(-1).values).float().mean().item()
+    print(f"   expert-set agreement on {len(sub)} tokens: {set_agree:.5f}")
+    assert set_agree >= 0.999
+    torch.testing.assert_close(y.view(-1, H)[sub.to(device)].float().cpu(), want.view(-1, H).float(), rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(gates.cpu()[sub].float(), want_g.float(), rtol=2e-2, atol=2e-2)
