@@ -363,17 +363,26 @@ __global__ __launch_bounds__(kGemmThreads, 1) void gemm_nt_dma_kernel(const Gemm
     b_src[p] = base + ((int64_t)col * g.K + c * 8) * 2;
   }
 
-  auto issue_tile = [&](int kt) {
+  const int wave_s = __builtin_amdgcn_readfirstlane(wave);   // scalar copy: LDS destinations stay in SGPRs
+  // one quarter (part 0..3) of a tile's LPT load instructions; parts are spread between MFMA
+  // groups so that their address set-up and issue never leave the matrix pipeline idle
+  auto issue_part = [&](int kt, int part) {
     uint8_t* st = lds + (kt % NS) * kStageBytes;
     const int koff = kt * kRow;
 #pragma unroll
-    for (int p = 0; p < PA; ++p)
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(a_src[p] + koff),
-                                       (__attribute__((address_space(3))) void*)(st + (4 * p + wave) * 1024), 16, 0, 0);
+    for (int q = 0; q < LPT; ++q) {
+      if ((q * 4) / LPT != part) continue;
+      if (q < PA)
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(a_src[q] + koff),
+                                         (__attribute__((address_space(3))) void*)(st + (4 * q + wave_s) * 1024), 16, 0, 0);
+      else
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(b_src[q - PA] + koff),
+                                         (__attribute__((address_space(3))) void*)(st + BM * kRow + (4 * (q - PA) + wave_s) * 1024), 16, 0, 0);
+    }
+  };
+  auto issue_tile = [&](int kt) {
 #pragma unroll
-    for (int p = 0; p < PB; ++p)
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(b_src[p] + koff),
-                                       (__attribute__((address_space(3))) void*)(st + BM * kRow + (4 * p + wave) * 1024), 16, 0, 0);
+    for (int part = 0; part < 4; ++part) issue_part(kt, part);
   };
 
   // fragment reads: lane reads row lane%32, logical chunk 2*slab + lane/32, into buffer slab&1
@@ -410,12 +419,16 @@ __global__ __launch_bounds__(kGemmThreads, 1) void gemm_nt_dma_kernel(const Gemm
   // slab `sl` of a tile while the fragments of the following slab are fetched.  The reads are
   // issued in the MIDDLE of the slab's MFMAs: the wait the compiler places in front of every
   // MFMA group covers all LDS reads, so they must be old by the time the next group starts.
-  auto slab_then_read = [&](int sl, int next_kt, int next_slab) {
+  // `fetch_kt` >= 0: also issue parts `part0` and `part0+1` of that tile's loads, one per MFMA group.
+  auto slab_then_read = [&](int sl, int next_kt, int next_slab, int fetch_kt = -1, int part0 = 0) {
     mfma_half(sl & 1, 0);
     __builtin_amdgcn_sched_barrier(0);
     read_frags(next_kt, next_slab);
+    if (fetch_kt >= 0) issue_part(fetch_kt, part0);
     __builtin_amdgcn_sched_barrier(0);
     mfma_half(sl & 1, 1);
+    __builtin_amdgcn_sched_barrier(0);
+    if (fetch_kt >= 0) issue_part(fetch_kt, part0 + 1);
     __builtin_amdgcn_sched_barrier(0);
   };
 
@@ -434,9 +447,11 @@ __global__ __launch_bounds__(kGemmThreads, 1) void gemm_nt_dma_kernel(const Gemm
   __builtin_amdgcn_s_barrier();
   OMNI_STAMP(1);
   read_frags(0, 0);
+  int fetch = -1;                             // tile whose loads are half issued (parts 0,1 done)
   for (int kt = 0; kt < num_kt - 1; ++kt) {
+    slab_then_read(0, kt, 1, fetch, 2);       // S >= 2: slab 0 is never the tile's last
 #pragma unroll
-    for (int sl = 0; sl < S - 1; ++sl) slab_then_read(sl, kt, sl + 1);
+    for (int sl = 1; sl < S - 1; ++sl) slab_then_read(sl, kt, sl + 1);
     wait_lds_reads();                         // this wave holds every fragment of tile kt
     // tiles kt+1 .. min(kt+NS-1, num_kt-1) are outstanding; tile kt+1 must have landed
     const int younger = num_kt - 2 - kt;
@@ -446,11 +461,12 @@ __global__ __launch_bounds__(kGemmThreads, 1) void gemm_nt_dma_kernel(const Gemm
 #ifndef OMNI_DBG_NO_BARRIER
     __builtin_amdgcn_s_barrier();             // tile kt+1 visible to all; stage of tile kt free
 #endif
-#ifndef OMNI_DBG_NO_DMA
-    if (kt + NS < num_kt) issue_tile(kt + NS);
+    fetch = (kt + NS < num_kt) ? kt + NS : -1;
+#ifdef OMNI_DBG_NO_DMA
+    fetch = -1;
 #endif
     __builtin_amdgcn_sched_barrier(0);
-    slab_then_read(S - 1, kt + 1, 0);
+    slab_then_read(S - 1, kt + 1, 0, fetch, 0);
   }
 #pragma unroll
   for (int sl = 0; sl < S - 1; ++sl) slab_then_read(sl, num_kt - 1, sl + 1);   // last tile
