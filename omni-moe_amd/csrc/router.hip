@@ -29,6 +29,60 @@ __device__ __forceinline__ bool goes_before(float sa, int pa, float sb, int pb) 
   return (sa > sb) || (sa == sb && pa < pb);
 }
 
+// Value of lane (lane ^ STRIDE) without touching LDS memory: DPP quad permutes (1, 2), two
+// bank-masked DPP row shifts (4, 8), a ds_swizzle bit pattern (16), v_permlane32_swap (32).
+template <int STRIDE>
+__device__ __forceinline__ int xor_lane_i(int v, int lane) {
+  if constexpr (STRIDE == 1) return __builtin_amdgcn_update_dpp(v, v, 0xB1, 0xf, 0xf, false);
+  else if constexpr (STRIDE == 2) return __builtin_amdgcn_update_dpp(v, v, 0x4E, 0xf, 0xf, false);
+  else if constexpr (STRIDE == 4) {
+    const int t = __builtin_amdgcn_update_dpp(v, v, 0x104, 0xf, 0x5, false);     // row_shl:4 into banks 0,2
+    return __builtin_amdgcn_update_dpp(t, v, 0x114, 0xf, 0xA, false);            // row_shr:4 into banks 1,3
+  } else if constexpr (STRIDE == 8) {
+    const int t = __builtin_amdgcn_update_dpp(v, v, 0x108, 0xf, 0x3, false);     // row_shl:8 into banks 0,1
+    return __builtin_amdgcn_update_dpp(t, v, 0x118, 0xf, 0xC, false);            // row_shr:8 into banks 2,3
+  } else if constexpr (STRIDE == 16) return __builtin_amdgcn_ds_swizzle(v, 0x401F);
+  else {
+    const auto sw = __builtin_amdgcn_permlane32_swap(v, v, false, false);         // [lo,lo] and [hi,hi]
+    return (lane & 32) ? (int)sw[0] : (int)sw[1];
+  }
+}
+template <int STRIDE>
+__device__ __forceinline__ float xor_lane_f(float v, int lane) {
+  return __int_as_float(xor_lane_i<STRIDE>(__float_as_int(v), lane));
+}
+
+// Compare-exchange step with a compile-time lane distance, fully unrolled (small R only).
+template <int R, int SIZE, int STRIDE>
+__device__ __forceinline__ void lane_stage_ct(float (&s)[R], int (&p)[R], const int lane) {
+#pragma unroll
+  for (int a = 0; a < R; ++a) {
+    const float os = xor_lane_f<STRIDE>(s[a], lane);
+    const int op = xor_lane_i<STRIDE>(p[a], lane);
+    const bool up = (((a * kWave) | lane) & SIZE) == 0;
+    const bool lower = (lane & STRIDE) == 0;
+    const bool take_other = (lower == up) != goes_before(s[a], p[a], os, op);
+    s[a] = take_other ? os : s[a];
+    p[a] = take_other ? op : p[a];
+  }
+}
+// strides STRIDE, STRIDE/2, ..., 1 of the merge for block size SIZE, on NL lists in lockstep
+template <int R, int SIZE, int STRIDE>
+__device__ __forceinline__ void lane_stages_ct(float (&s0)[R], int (&p0)[R], float (&s1)[R], int (&p1)[R], const int lane, const bool two) {
+  if constexpr (STRIDE >= 1) {
+    lane_stage_ct<R, SIZE, STRIDE>(s0, p0, lane);
+    if (two) lane_stage_ct<R, SIZE, STRIDE>(s1, p1, lane);
+    lane_stages_ct<R, SIZE, STRIDE / 2>(s0, p0, s1, p1, lane, two);
+  }
+}
+template <int R, int SIZE>
+__device__ __forceinline__ void small_sizes_ct(float (&s0)[R], int (&p0)[R], float (&s1)[R], int (&p1)[R], const int lane, const bool two) {
+  if constexpr (SIZE <= kWave) {
+    lane_stages_ct<R, SIZE, SIZE / 2>(s0, p0, s1, p1, lane, two);
+    small_sizes_ct<R, SIZE * 2>(s0, p0, s1, p1, lane, two);
+  }
+}
+
 // One compare-exchange step between lanes `stride` apart (stride < 64), all R registers.
 template <int R>
 __device__ __forceinline__ void lane_stage(float (&s)[R], int (&p)[R], const int lane, const int size, const int stride) {
@@ -72,12 +126,18 @@ __device__ __forceinline__ void reg_stages_down(float (&s)[R], int (&p)[R]) {
 }
 
 // Merge steps for block size SIZE (> 64) and the sizes above it, up to 64*R.
+constexpr int kUnrollMaxR = 2;     // lists of <= 128 items use the unrolled, LDS-free exchanges
+
 template <int R, int SIZE>
 __device__ __forceinline__ void big_sizes(float (&s)[R], int (&p)[R], const int lane) {
   if constexpr (SIZE <= kWave * R) {
     reg_stages_down<R, SIZE, SIZE / (2 * kWave)>(s, p);
+    if constexpr (R <= kUnrollMaxR) {
+      lane_stages_ct<R, SIZE, kWave / 2>(s, p, s, p, lane, false);
+    } else {
 #pragma nounroll
-    for (int stride = kWave / 2; stride >= 1; stride >>= 1) lane_stage<R>(s, p, lane, SIZE, stride);
+      for (int stride = kWave / 2; stride >= 1; stride >>= 1) lane_stage<R>(s, p, lane, SIZE, stride);
+    }
     big_sizes<R, SIZE * 2>(s, p, lane);
   }
 }
@@ -87,10 +147,14 @@ __device__ __forceinline__ void big_sizes(float (&s)[R], int (&p)[R], const int 
 // value); steps between registers are unrolled so that register indices are constants.
 template <int R>
 __device__ __forceinline__ void bitonic_sort(float (&s)[R], int (&p)[R], const int lane) {
+  if constexpr (R <= kUnrollMaxR) {
+    small_sizes_ct<R, 2>(s, p, s, p, lane, false);
+  } else {
 #pragma nounroll
-  for (int size = 2; size <= kWave; size <<= 1) {
+    for (int size = 2; size <= kWave; size <<= 1) {
 #pragma nounroll
-    for (int stride = size >> 1; stride >= 1; stride >>= 1) lane_stage<R>(s, p, lane, size, stride);
+      for (int stride = size >> 1; stride >= 1; stride >>= 1) lane_stage<R>(s, p, lane, size, stride);
+    }
   }
   big_sizes<R, 2 * kWave>(s, p, lane);
 }
@@ -102,22 +166,30 @@ __device__ __forceinline__ void big_sizes2(float (&s0)[R], int (&p0)[R], float (
   if constexpr (SIZE <= kWave * R) {
     reg_stages_down<R, SIZE, SIZE / (2 * kWave)>(s0, p0);
     reg_stages_down<R, SIZE, SIZE / (2 * kWave)>(s1, p1);
+    if constexpr (R <= kUnrollMaxR) {
+      lane_stages_ct<R, SIZE, kWave / 2>(s0, p0, s1, p1, lane, true);
+    } else {
 #pragma nounroll
-    for (int stride = kWave / 2; stride >= 1; stride >>= 1) {
-      lane_stage<R>(s0, p0, lane, SIZE, stride);
-      lane_stage<R>(s1, p1, lane, SIZE, stride);
+      for (int stride = kWave / 2; stride >= 1; stride >>= 1) {
+        lane_stage<R>(s0, p0, lane, SIZE, stride);
+        lane_stage<R>(s1, p1, lane, SIZE, stride);
+      }
     }
     big_sizes2<R, SIZE * 2>(s0, p0, s1, p1, lane);
   }
 }
 template <int R>
 __device__ __forceinline__ void bitonic_sort2(float (&s0)[R], int (&p0)[R], float (&s1)[R], int (&p1)[R], const int lane) {
+  if constexpr (R <= kUnrollMaxR) {
+    small_sizes_ct<R, 2>(s0, p0, s1, p1, lane, true);
+  } else {
 #pragma nounroll
-  for (int size = 2; size <= kWave; size <<= 1) {
+    for (int size = 2; size <= kWave; size <<= 1) {
 #pragma nounroll
-    for (int stride = size >> 1; stride >= 1; stride >>= 1) {
-      lane_stage<R>(s0, p0, lane, size, stride);
-      lane_stage<R>(s1, p1, lane, size, stride);
+      for (int stride = size >> 1; stride >= 1; stride >>= 1) {
+        lane_stage<R>(s0, p0, lane, size, stride);
+        lane_stage<R>(s1, p1, lane, size, stride);
+      }
     }
   }
   big_sizes2<R, 2 * kWave>(s0, p0, s1, p1, lane);
