@@ -233,6 +233,7 @@ struct SelectArgs {
   void* gates;           // [T,k] storage dtype = exp(score), may be NULL
   int32_t* indices;      // [T,k]
   int num_tokens, r, k, kp, dt;
+  uint8_t row_cells[128]; // candidate cells in row a: min(kp, k/(a+1)), filled by select_dispatch
 };
 
 // BatchNorm (affine-free) then log-softmax of one half, in place: v holds the raw projection
@@ -269,14 +270,15 @@ __global__ __launch_bounds__(kRouterWaves* kWave) void router_select_kernel(cons
   // with min(kp, k/(a+1)) cells each.  Payload (a<<8)|b orders like position a*kp+b.
   int cell[C];
 #pragma unroll
-  for (int c = 0; c < C; ++c) {
-    int ci = c * kWave + lane, a = 0;
-    cell[c] = -1;
-    for (; a < kp; ++a) {
-      const int cnt = min(kp, k / (a + 1));
-      if (ci < cnt) { cell[c] = (a << 8) | ci; break; }
-      ci -= cnt;
+  for (int c = 0; c < C; ++c) cell[c] = -1;
+  for (int a = 0, start = 0; a < kp; ++a) {       // uniform loop, counts come with the arguments
+    const int cnt = g.row_cells[a];
+#pragma unroll
+    for (int c = 0; c < C; ++c) {
+      const int b = c * kWave + lane - start;
+      cell[c] = (unsigned)b < (unsigned)cnt ? (a << 8) | b : cell[c];
     }
+    start += cnt;
   }
 
   for (int t = wave; t < g.num_tokens; t += num_waves) {
@@ -325,6 +327,171 @@ __global__ __launch_bounds__(kRouterWaves* kWave) void router_select_kernel(cons
   }
 }
 
+// ---- 16-bit scores: (score, payload) packed into one ordered 32-bit key ---------------------
+// key = order-preserving image of the 16-bit score << 16 | (0xFFFF - payload): a larger key goes
+// first, equal scores resolve to the lower payload, and a compare-exchange is one max / min.
+// Four times fewer VALU instructions than the (float, int) pairs the fp32 path needs.
+__device__ __forceinline__ uint32_t ord16(uint32_t bits) { return bits ^ ((bits & 0x8000u) ? 0xFFFFu : 0x8000u); }
+__device__ __forceinline__ uint32_t unord16(uint32_t u) { return u ^ ((u & 0x8000u) ? 0x8000u : 0xFFFFu); }
+__device__ __forceinline__ uint32_t make_key(float v, int payload, int dt) {      // v is representable in dt
+  v += 0.0f;                                                                      // -0 -> +0: they compare equal as floats
+  const uint32_t bits = dt == kBF16 ? (uint32_t)f32_to_bf16_bits(v) : (uint32_t)f32_to_f16_bits(v);
+  return (ord16(bits) << 16) | (0xFFFFu - (uint32_t)payload);
+}
+__device__ __forceinline__ float key_score(uint32_t key, int dt) {
+  const uint32_t bits = unord16(key >> 16);
+  return dt == kBF16 ? bf16_bits_to_f32((uint16_t)bits) : f16_bits_to_f32((uint16_t)bits);
+}
+__device__ __forceinline__ int key_payload(uint32_t key) { return (int)(0xFFFFu - (key & 0xFFFFu)); }
+
+template <int R, int SIZE, int STRIDE>
+__device__ __forceinline__ void kstage_ct(uint32_t (&k)[R], const int lane) {
+#pragma unroll
+  for (int a = 0; a < R; ++a) {
+    const uint32_t o = (uint32_t)xor_lane_i<STRIDE>((int)k[a], lane);
+    const bool up = (((a * kWave) | lane) & SIZE) == 0, lower = (lane & STRIDE) == 0;
+    k[a] = (lower == up) ? max(k[a], o) : min(k[a], o);
+  }
+}
+template <int R>
+__device__ __forceinline__ void kstage_rt(uint32_t (&k)[R], const int lane, const int size, const int stride) {
+#pragma unroll
+  for (int a = 0; a < R; ++a) {
+    const uint32_t o = (uint32_t)__shfl_xor((int)k[a], stride, kWave);
+    const bool up = (((a * kWave) | lane) & size) == 0, lower = (lane & stride) == 0;
+    k[a] = (lower == up) ? max(k[a], o) : min(k[a], o);
+  }
+}
+template <int R, int SIZE, int RS>
+__device__ __forceinline__ void kreg_stages(uint32_t (&k)[R]) {
+  if constexpr (RS >= 1) {
+#pragma unroll
+    for (int a = 0; a < R; ++a) {
+      if ((a & RS) == 0) {
+        const int b = a | RS;
+        const bool up = ((a * kWave) & SIZE) == 0;
+        const uint32_t hi = max(k[a], k[b]), lo = min(k[a], k[b]);
+        k[a] = up ? hi : lo;
+        k[b] = up ? lo : hi;
+      }
+    }
+    kreg_stages<R, SIZE, RS / 2>(k);
+  }
+}
+// lane distances STRIDE..1 of the merge for block size SIZE, on one or two lists
+template <int R, int SIZE, int STRIDE>
+__device__ __forceinline__ void kstages_ct(uint32_t (&k0)[R], uint32_t (&k1)[R], const int lane, const bool two) {
+  if constexpr (STRIDE >= 1) {
+    kstage_ct<R, SIZE, STRIDE>(k0, lane);
+    if (two) kstage_ct<R, SIZE, STRIDE>(k1, lane);
+    kstages_ct<R, SIZE, STRIDE / 2>(k0, k1, lane, two);
+  }
+}
+template <int R, int SIZE>
+__device__ __forceinline__ void ksizes(uint32_t (&k0)[R], uint32_t (&k1)[R], const int lane, const bool two) {
+  if constexpr (SIZE <= kWave * R) {
+    if constexpr (SIZE > kWave) {
+      kreg_stages<R, SIZE, SIZE / (2 * kWave)>(k0);
+      if (two) kreg_stages<R, SIZE, SIZE / (2 * kWave)>(k1);
+    }
+    constexpr int kFirst = SIZE > kWave ? kWave / 2 : SIZE / 2;
+    if constexpr (R <= kUnrollMaxR) {
+      kstages_ct<R, SIZE, kFirst>(k0, k1, lane, two);
+    } else {
+#pragma nounroll
+      for (int stride = kFirst; stride >= 1; stride >>= 1) {
+        kstage_rt<R>(k0, lane, SIZE, stride);
+        if (two) kstage_rt<R>(k1, lane, SIZE, stride);
+      }
+    }
+    ksizes<R, SIZE * 2>(k0, k1, lane, two);
+  }
+}
+// sorts the 64*R keys of each list descending (item e = reg*64 + lane)
+template <int R> __device__ __forceinline__ void ksort(uint32_t (&k)[R], const int lane) { ksizes<R, 2>(k, k, lane, false); }
+template <int R> __device__ __forceinline__ void ksort2(uint32_t (&k0)[R], uint32_t (&k1)[R], const int lane) { ksizes<R, 2>(k0, k1, lane, true); }
+
+template <int R>
+__device__ __forceinline__ uint32_t sorted_key(const uint32_t (&v)[R], int i) {
+  uint32_t r0 = (uint32_t)__shfl((int)v[0], i & 63, kWave);
+  if constexpr (R >= 2) {
+    const uint32_t r1 = (uint32_t)__shfl((int)v[1], i & 63, kWave);
+    r0 = (i >= kWave) ? r1 : r0;
+  }
+  return r0;
+}
+
+// Same selection as router_select_kernel for bf16 / f16 storage, on packed keys.
+template <int R, int C>
+__global__ __launch_bounds__(kRouterWaves* kWave) void router_select_packed_kernel(const SelectArgs g) {
+  const int lane = lane_id();
+  const int wave = blockIdx.x * kRouterWaves + (threadIdx.x >> 6);
+  const int num_waves = gridDim.x * kRouterWaves;
+  const int r = g.r, k = g.k, kp = g.kp, dt = g.dt;
+
+  int cell[C];                                  // as in router_select_kernel
+#pragma unroll
+  for (int c = 0; c < C; ++c) cell[c] = -1;
+  for (int a = 0, start = 0; a < kp; ++a) {       // uniform loop, counts come with the arguments
+    const int cnt = g.row_cells[a];
+#pragma unroll
+    for (int c = 0; c < C; ++c) {
+      const int b = c * kWave + lane - start;
+      cell[c] = (unsigned)b < (unsigned)cnt ? (a << 8) | b : cell[c];
+    }
+    start += cnt;
+  }
+
+  for (int t = wave; t < g.num_tokens; t += num_waves) {
+    float sx[R], sy[R];
+#pragma unroll
+    for (int a = 0; a < R; ++a) {
+      const int key = a * kWave + lane;
+      const bool ok = key < r;
+      sx[a] = ok ? load_score(g.lx, int64_t(t) * g.row_stride + key, dt) : kNegInf;
+      sy[a] = ok ? load_score(g.ly, int64_t(t) * g.row_stride + key, dt) : kNegInf;
+    }
+    if (g.stats) {
+      normalise_half<R>(sx, g.stats, g.stats + r, r, lane, dt);
+      normalise_half<R>(sy, g.stats + 2 * r, g.stats + 3 * r, r, lane, dt);
+    }
+    uint32_t kx[R], ky[R];
+#pragma unroll
+    for (int a = 0; a < R; ++a) {
+      const int key = a * kWave + lane;
+      kx[a] = key < r ? make_key(sx[a], key, dt) : 0u;          // 0 sorts behind every real key
+      ky[a] = key < r ? make_key(sy[a], key, dt) : 0u;
+    }
+    ksort2<R>(kx, ky, lane);
+
+    uint32_t ck[C];
+#pragma unroll
+    for (int c = 0; c < C; ++c) {
+      const bool ok = cell[c] >= 0;
+      const int a = ok ? (cell[c] >> 8) : 0, b = ok ? (cell[c] & 255) : 0;
+      const float va = key_score(sorted_key<R>(kx, a), dt), vb = key_score(sorted_key<R>(ky, b), dt);
+      ck[c] = ok ? make_key(round_score(va + vb, dt), cell[c], dt) : 0u;
+    }
+    ksort<C>(ck, lane);
+
+    constexpr int kOut = (C >= 2) ? 2 : 1;          // k <= 128 -> winners live in regs 0..1
+#pragma unroll
+    for (int c = 0; c < kOut; ++c) {
+      const int j = c * kWave + lane;
+      const bool ok = j < k;
+      const int pl = ok ? key_payload(ck[c]) : 0;
+      const int ia = key_payload(sorted_key<R>(kx, pl >> 8)), ib = key_payload(sorted_key<R>(ky, pl & 255));
+      if (ok) {
+        const int64_t o = int64_t(t) * k + j;
+        const float sc = key_score(ck[c], dt);
+        if (g.scores) store_score(g.scores, o, sc, dt);
+        if (g.gates) store_score(g.gates, o, expf(sc), dt);         // gate = P(x key) * P(y key)
+        g.indices[o] = ia * r + ib;
+      }
+    }
+  }
+}
+
 static int num_cells(int k, int kp) {
   int n = 0;
   for (int a = 0; a < kp; ++a) n += (kp < k / (a + 1)) ? kp : k / (a + 1);
@@ -335,7 +502,10 @@ template <int R, int C>
 static hipError_t launch_select(const SelectArgs& g, hipStream_t s) {
   int64_t blocks = ((int64_t)g.num_tokens + kRouterWaves - 1) / kRouterWaves;
   if (blocks > 256 * 16) blocks = 256 * 16;     // waves loop over tokens beyond that
-  hipLaunchKernelGGL((router_select_kernel<R, C>), dim3((unsigned)blocks), dim3(kRouterWaves * kWave), 0, s, g);
+  if (g.dt == kF32)
+    hipLaunchKernelGGL((router_select_kernel<R, C>), dim3((unsigned)blocks), dim3(kRouterWaves * kWave), 0, s, g);
+  else
+    hipLaunchKernelGGL((router_select_packed_kernel<R, C>), dim3((unsigned)blocks), dim3(kRouterWaves * kWave), 0, s, g);
   return hipGetLastError();
 }
 
@@ -350,6 +520,7 @@ static hipError_t select_by_cells(int cpl, const SelectArgs& g, hipStream_t s) {
 
 static int select_dispatch(SelectArgs g, hipStream_t s) {
   g.kp = g.r < g.k ? g.r : g.k;
+  for (int a = 0; a < 128; ++a) g.row_cells[a] = a < g.kp ? (uint8_t)(g.kp < g.k / (a + 1) ? g.kp : g.k / (a + 1)) : 0;
   const int cpl = (num_cells(g.k, g.kp) + kWave - 1) / kWave;   // <= 11 for k <= 128
   const int rpl = (g.r + kWave - 1) / kWave;
   hipError_t err;
