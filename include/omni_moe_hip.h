@@ -73,8 +73,9 @@ OMNI_API int32_t omni_router_select(const void* logits_x, const void* logits_y, 
  *   offsets          : device [num_experts+1] int32; pairs of expert e occupy
  *                      [offsets[e], offsets[e+1]) of the sorted arrays
  *   sorted_pair_ids  : device [num_tokens*k] int32, pair id = token*k + slot;
- *                      inside a segment the order is unspecified (as with the
- *                      reference's torch.sort, :71)
+ *                      inside a segment ascending (a stable sort; the reference's
+ *                      torch.sort, :71, leaves that order open); pairs whose id is
+ *                      outside [0, N) follow at positions >= offsets[N]
  *   sorted_token_ids : device [num_tokens*k] int32 (= sorted_pair_ids / k), may be NULL
  *   workspace        : device, omni_schedule_workspace_bytes() bytes */
 OMNI_API size_t omni_schedule_workspace_bytes(int64_t num_tokens, int32_t num_experts_per_token, int64_t num_experts);

@@ -239,10 +239,7 @@ def test_layer_config5_large_skewed(device):
     ids_c = ids.cpu()
     want_off, want_pairs, _ = oracle.schedule(ids_c, N)
     assert torch.equal(sched.offsets.cpu(), want_off)
-    flat = ids_c.reshape(-1).long()
-    pairs = sched.sorted_pair_ids.cpu().long()
-    assert torch.equal(flat[pairs], flat[want_pairs.long()])
-    assert torch.equal(torch.sort(pairs).values, torch.arange(T * k))
+    assert torch.equal(sched.sorted_pair_ids.cpu(), want_pairs)
     seg = (want_off[1:] - want_off[:-1]).float()
     print(f"   pairs per expert: max {int(seg.max())}, mean over used {seg[seg > 0].mean():.1f}, used experts {int((seg > 0).sum())}")
     assert seg.max() > 100 * seg[seg > 0].mean()          # the skew is there

@@ -89,7 +89,8 @@ def test_router_select_contract(device):
 
 # ---------------------------------------------------------------- schedule
 SCHED_CASES = [(512, 8, 1024, "uniform"), (4096, 16, 4096, "uniform"), (16384, 16, 4096, "uniform"),
-               (4096, 32, 262144, "zipf"), (1000, 6, 5000, "zipf"), (3, 2, 7, "uniform"), (2048, 16, 64, "hot")]
+               (4096, 32, 262144, "zipf"), (1000, 6, 5000, "zipf"), (3, 2, 7, "uniform"), (2048, 16, 64, "hot"),
+               (32768, 32, 262144, "zipf"), (777, 10, 1048576, "uniform"), (100, 4, 1, "hot"), (5000, 8, 4097, "uniform")]
 
 
 def _sched_ids(T, k, N, kind, seed):
@@ -112,14 +113,10 @@ def test_schedule_matches_oracle(case, device):
     torch.cuda.synchronize()
     off, pairs, tok = got.offsets.cpu(), got.sorted_pair_ids.cpu(), got.sorted_token_ids.cpu()
     assert torch.equal(off, want_off)
-    # the pairs are a permutation, grouped by expert; inside a segment the order is free
-    # (as with the reference's torch.sort) -> compare after ordering each segment
-    flat = ids.reshape(-1).long()
-    assert torch.equal(flat[pairs.long()], flat[want_pairs.long()])
-    key = flat[pairs.long()] * (T * k) + pairs.long()
-    canon = pairs[torch.argsort(key)]
-    assert torch.equal(canon, want_pairs)
+    assert torch.equal(pairs, want_pairs)                  # stable: bit-exact against torch.sort(stable=True)
     assert torch.equal(tok, (pairs // k).to(torch.int32))
+    again = _ops().hip_omni_schedule_func(ids.to(device), N)
+    assert torch.equal(again.sorted_pair_ids.cpu(), pairs)  # and identical from run to run
 
 
 # ---------------------------------------------------------------- expert
@@ -185,3 +182,20 @@ def test_expert_edge_cases(device):
     torch.testing.assert_close(y3.float(), y1.float(), rtol=2e-2, atol=1e-3)                     # slot order is free
     with pytest.raises(ValueError):
         hip.hip_omni_expert_func(x, up, down[:, :128], gates, ids)
+
+
+def test_schedule_drops_out_of_range_ids(device):
+    g = torch.Generator().manual_seed(9)
+    T, k, N = 300, 6, 50
+    ids = torch.randint(-3, N + 5, (T, k), generator=g, dtype=torch.int32)
+    got = _ops().hip_omni_schedule_func(ids.to(device), N)
+    flat = ids.reshape(-1)
+    valid = (flat >= 0) & (flat < N)
+    want_off = torch.zeros(N + 1, dtype=torch.int64)
+    want_off[1:] = torch.cumsum(torch.bincount(flat[valid].long(), minlength=N), 0)
+    assert torch.equal(got.offsets.cpu().long(), want_off)
+    nv = int(valid.sum())
+    pairs = got.sorted_pair_ids.cpu().long()
+    order = torch.sort(torch.where(valid, flat, torch.full_like(flat, N)).long(), stable=True).indices
+    assert torch.equal(pairs[:nv], order[:nv])
+    assert torch.equal(torch.sort(pairs).values, torch.arange(T * k))       # still a permutation
