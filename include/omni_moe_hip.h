@@ -90,7 +90,9 @@ OMNI_API int32_t omni_schedule(const int32_t* indices, int32_t* offsets, int32_t
  *   indices [T,k] int32 in [0,N) (duplicates inside a token add; not range-checked,
  *   as in the reference); y [T,H] dtype `dtype`, fully overwritten.
  * H*sizeof(elem) must be a multiple of 16.  Sums are fp32, one rounding at the end.
- *   algo      : OMNI_EXPERT_ALGO_*
+ *   algo      : OMNI_EXPERT_ALGO_* (AUTO = GATHER).  SEGMENT is the expert-centric organisation:
+ *               omni_schedule, a pass over the sorted pairs for the coefficients, a token pass
+ *               for the sum; same results, kept so that both can be measured.
  *   workspace : omni_expert_workspace_bytes() bytes (0 for GATHER: may be NULL) */
 OMNI_API size_t omni_expert_workspace_bytes(int64_t num_tokens, int32_t hidden_size, int64_t num_experts,
                                    int32_t num_experts_per_token, int32_t dtype, int32_t algo);

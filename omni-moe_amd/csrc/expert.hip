@@ -10,6 +10,17 @@
 // and the gate-weighted down rows accumulate in fp32 registers.  Nothing but y
 // is written: no score buffer, no atomics, and the summation order is fixed
 // (slot 0..k-1), so results are run-to-run identical.
+//
+// Expert-centric variant ("segment" algorithm), the reference's own organisation
+// (omni_expert.py:8-168): the pairs are first grouped by expert (omni_schedule), then
+//   A. waves walk the sorted pair list, 16 consecutive pairs each -- so a popular expert's
+//      segment is spread over many waves and an unpopular one costs one short visit -- gather
+//      the pair's x row and its expert's up row (which repeats along a segment and therefore
+//      hits in cache), and write the coefficient silu(<x,u>)*g of the pair;
+//   B. a token-resident pass accumulates coefficient * down row into y, in slot order.
+// No atomics, same fixed summation order as the gather algorithm, hence identical results;
+// it moves the same rows plus the schedule and a [T,k] fp32 coefficient buffer, and exists so
+// that the two organisations can be measured side by side.
 #include "common.h"
 #include "omni_moe_hip.h"
 
@@ -31,9 +42,7 @@ __device__ __forceinline__ float dot16(const u32x4_t a, const u32x4_t b, float a
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const uint32_t ai = a[i], bi = b[i];
-      f16x2_t p = __builtin_bit_cast(f16x2_t, ai), q = __builtin_bit_cast(f16x2_t, bi);
-      acc = fmaf(float(p[0]), float(q[0]), acc);
-      acc = fmaf(float(p[1]), float(q[1]), acc);
+      acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2_t, ai), __builtin_bit_cast(f16x2_t, bi), acc, false);
     }
   } else {
 #pragma unroll
@@ -187,12 +196,150 @@ static int expert_gather_dispatch(const void* x, const void* up, const void* dow
   return err == hipSuccess ? OMNI_OK : OMNI_ERR_HIP_BASE + (int)err;
 }
 
+// ---- expert-centric variant -------------------------------------------------------------------
+constexpr int kPairsPerWave = 16;
+
+template <int DT, int NCH>
+__global__ __launch_bounds__(256, 2) void expert_segment_scores_kernel(
+    const uint8_t* __restrict__ x, const uint8_t* __restrict__ up, const void* __restrict__ gates,
+    const int32_t* __restrict__ ids, const int32_t* __restrict__ sorted_pair_ids, const int32_t* __restrict__ offsets,
+    float* __restrict__ coef, int hidden, int top_k, int64_t num_experts) {
+  constexpr int E = Row16<DT>::kElems;
+  constexpr int G = (NCH <= 2) ? 8 : (NCH <= 4 ? 4 : 2);       // pairs whose rows are in flight together
+  const int lane = lane_id();
+  const int num_valid = offsets[num_experts];                   // pairs with an id inside the table
+  const int wave = __builtin_amdgcn_readfirstlane(blockIdx.x * 4 + (threadIdx.x >> 6));
+  const int pos0 = wave * kPairsPerWave;
+  if (pos0 >= num_valid) return;
+  const int64_t row_bytes = int64_t(hidden) * (16 / E);
+  bool live[NCH];
+  int64_t off[NCH];
+#pragma unroll
+  for (int c = 0; c < NCH; ++c) {
+    live[c] = (c * kWave + lane) * E < hidden;
+    off[c] = int64_t(c * kWave + lane) * 16;
+  }
+  for (int g0 = 0; g0 < kPairsPerWave; g0 += G) {
+    int pid[G];
+    bool ok[G];
+    u32x4_t xr[G][NCH], ur[G][NCH];
+#pragma unroll
+    for (int i = 0; i < G; ++i) {
+      const int pos = pos0 + g0 + i;
+      ok[i] = pos < num_valid;
+      pid[i] = sorted_pair_ids[ok[i] ? pos : pos0];
+      const int t = pid[i] / top_k, e = ids[pid[i]];
+#pragma unroll
+      for (int c = 0; c < NCH; ++c) {
+        xr[i][c] = live[c] ? *(const u32x4_t*)(x + t * row_bytes + off[c]) : u32x4_t{0, 0, 0, 0};
+        ur[i][c] = live[c] ? *(const u32x4_t*)(up + e * row_bytes + off[c]) : u32x4_t{0, 0, 0, 0};
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < G; ++i) {
+      float p = 0.f;
+#pragma unroll
+      for (int c = 0; c < NCH; ++c) p = dot16<DT>(xr[i][c], ur[i][c], p);
+      const float sdot = wave_sum(p);
+      if (ok[i] && lane == 0) coef[pid[i]] = silu_f32(sdot) * Elem<DT>::load(gates, pid[i]);
+    }
+  }
+}
+
+// y[t] = sum_j coef[t,j] * down[id[t,j]] in slot order; coef comes from the scores pass.
+template <int DT, int NCH, int G>
+__global__ __launch_bounds__(kTokensPerBlock* kWave, 2) void expert_accumulate_kernel(
+    const uint8_t* __restrict__ down, const float* __restrict__ coef, const int32_t* __restrict__ ids,
+    uint8_t* __restrict__ y, int num_tokens, int hidden, int top_k, uint32_t num_experts) {
+  constexpr int E = Row16<DT>::kElems;
+  const int lane = lane_id();
+  const int t = __builtin_amdgcn_readfirstlane(blockIdx.x * kTokensPerBlock + (threadIdx.x >> 6));
+  if (t >= num_tokens) return;
+  const int64_t row_bytes = int64_t(hidden) * (16 / E);
+  bool live[NCH];
+  int64_t off[NCH];
+  float acc[NCH][E];
+#pragma unroll
+  for (int c = 0; c < NCH; ++c) {
+    live[c] = (c * kWave + lane) * E < hidden;
+    off[c] = int64_t(c * kWave + lane) * 16;
+#pragma unroll
+    for (int i = 0; i < E; ++i) acc[c][i] = 0.f;
+  }
+  for (int j0 = 0; j0 < top_k; j0 += G) {
+    float cf[G];
+    u32x4_t vr[G][NCH];
+#pragma unroll
+    for (int i = 0; i < G; ++i) {
+      const int j = min(j0 + i, top_k - 1);
+      const int id = ids[int64_t(t) * top_k + j];
+      const bool ok = (j0 + i < top_k) && (uint32_t)id < num_experts;
+      cf[i] = ok ? coef[int64_t(t) * top_k + j] : 0.f;
+      const int e = ok ? id : 0;
+#pragma unroll
+      for (int c = 0; c < NCH; ++c)
+        vr[i][c] = live[c] ? *(const u32x4_t*)(down + e * row_bytes + off[c]) : u32x4_t{0, 0, 0, 0};
+    }
+#pragma unroll
+    for (int i = 0; i < G; ++i)
+#pragma unroll
+      for (int c = 0; c < NCH; ++c) axpy16<DT>(cf[i], vr[i][c], acc[c]);
+  }
+#pragma unroll
+  for (int c = 0; c < NCH; ++c)
+    if (live[c]) *(u32x4_t*)(y + t * row_bytes + off[c]) = pack16<DT>(acc[c]);
+}
+
+static inline size_t align256(size_t v) { return (v + 255) / 256 * 256; }
+
+template <int DT, int NCH, int G>
+static hipError_t launch_segment(const void* x, const void* up, const void* down, const void* gates, const int32_t* ids,
+                                 const int32_t* sorted_pair_ids, const int32_t* offsets, float* coef, void* y, int64_t T,
+                                 int H, int k, int64_t N, hipStream_t s) {
+  const int64_t P = T * k;
+  const unsigned waves = (unsigned)((P + kPairsPerWave - 1) / kPairsPerWave);
+  hipLaunchKernelGGL((expert_segment_scores_kernel<DT, NCH>), dim3((waves + 3) / 4), dim3(256), 0, s, (const uint8_t*)x,
+                     (const uint8_t*)up, gates, ids, sorted_pair_ids, offsets, coef, H, k, N);
+  hipLaunchKernelGGL((expert_accumulate_kernel<DT, NCH, G>), dim3((unsigned)((T + kTokensPerBlock - 1) / kTokensPerBlock)),
+                     dim3(kTokensPerBlock * kWave), 0, s, (const uint8_t*)down, coef, ids, (uint8_t*)y, (int)T, H, k, (uint32_t)N);
+  return hipGetLastError();
+}
+
+// workspace: offsets [N+1] | sorted pair ids [P] | coefficients [P] f32 | schedule workspace
+template <int DT>
+static int expert_segment_dispatch(const void* x, const void* up, const void* down, const void* gates, const int32_t* ids,
+                                   void* y, int64_t T, int H, int k, int64_t N, void* workspace, hipStream_t s) {
+  constexpr int E = Row16<DT>::kElems;
+  if (H % E != 0) return OMNI_ERR_SHAPE;
+  if (T == 0) return OMNI_OK;
+  if (k == 0) return expert_gather_dispatch<DT>(x, up, down, gates, ids, y, T, H, k, N, s);   // writes zeros
+  if (!workspace) return OMNI_ERR_WORKSPACE;
+  const int64_t P = T * k;
+  char* w = (char*)workspace;
+  int32_t* offsets = (int32_t*)w;          w += align256((size_t)(N + 1) * 4);
+  int32_t* sorted_pair_ids = (int32_t*)w;  w += align256((size_t)P * 4);
+  float* coef = (float*)w;                 w += align256((size_t)P * 4);
+  if (int e = omni_schedule(ids, offsets, sorted_pair_ids, nullptr, T, k, N, w, s)) return e;
+  const int nch = (H + kWave * E - 1) / (kWave * E);
+  hipError_t err;
+  if (nch <= 1) err = launch_segment<DT, 1, 16>(x, up, down, gates, ids, sorted_pair_ids, offsets, coef, y, T, H, k, N, s);
+  else if (nch <= 2) err = launch_segment<DT, 2, 8>(x, up, down, gates, ids, sorted_pair_ids, offsets, coef, y, T, H, k, N, s);
+  else if (nch <= 4) err = launch_segment<DT, 4, 4>(x, up, down, gates, ids, sorted_pair_ids, offsets, coef, y, T, H, k, N, s);
+  else if (nch <= 8) err = launch_segment<DT, 8, 2>(x, up, down, gates, ids, sorted_pair_ids, offsets, coef, y, T, H, k, N, s);
+  else return OMNI_ERR_UNSUPPORTED;
+  return err == hipSuccess ? OMNI_OK : OMNI_ERR_HIP_BASE + (int)err;
+}
+
 }  // namespace omni
 
 extern "C" OMNI_API size_t omni_expert_workspace_bytes(int64_t num_tokens, int32_t hidden_size, int64_t num_experts,
                                                        int32_t num_experts_per_token, int32_t dtype, int32_t algo) {
-  (void)num_tokens; (void)hidden_size; (void)num_experts; (void)num_experts_per_token; (void)dtype; (void)algo;
-  return 0;   // the gather algorithm keeps everything in registers
+  (void)hidden_size; (void)dtype;
+  if (algo != OMNI_EXPERT_ALGO_SEGMENT) return 0;   // the gather algorithm keeps everything in registers
+  if (num_tokens < 0 || num_experts <= 0 || num_experts_per_token < 0) return 0;
+  const size_t P = (size_t)num_tokens * (size_t)num_experts_per_token;
+  return omni::align256((size_t)(num_experts + 1) * 4) + 2 * omni::align256(P * 4) +
+         omni_schedule_workspace_bytes(num_tokens, num_experts_per_token, num_experts);
 }
 
 extern "C" OMNI_API int32_t omni_expert_fwd(const void* x, const void* up_weight, const void* down_weight,
@@ -206,7 +353,14 @@ extern "C" OMNI_API int32_t omni_expert_fwd(const void* x, const void* up_weight
   if (num_tokens > 0 && (!x || !up_weight || !down_weight || !y)) return OMNI_ERR_NULL;
   if (num_tokens > 0 && num_experts_per_token > 0 && (!routing_weights || !indices)) return OMNI_ERR_NULL;
   hipStream_t s = (hipStream_t)stream;
-  (void)workspace;
+  if (algo == OMNI_EXPERT_ALGO_SEGMENT) {
+    switch (dtype) {
+      case OMNI_BF16: return expert_segment_dispatch<kBF16>(x, up_weight, down_weight, routing_weights, indices, y, num_tokens, hidden_size, num_experts_per_token, num_experts, workspace, s);
+      case OMNI_F16: return expert_segment_dispatch<kF16>(x, up_weight, down_weight, routing_weights, indices, y, num_tokens, hidden_size, num_experts_per_token, num_experts, workspace, s);
+      case OMNI_F32: return expert_segment_dispatch<kF32>(x, up_weight, down_weight, routing_weights, indices, y, num_tokens, hidden_size, num_experts_per_token, num_experts, workspace, s);
+      default: return OMNI_ERR_DTYPE;
+    }
+  }
   if (algo != OMNI_EXPERT_ALGO_AUTO && algo != OMNI_EXPERT_ALGO_GATHER) return OMNI_ERR_UNSUPPORTED;
   switch (dtype) {
     case OMNI_BF16: return expert_gather_dispatch<kBF16>(x, up_weight, down_weight, routing_weights, indices, y, num_tokens, hidden_size, num_experts_per_token, num_experts, s);

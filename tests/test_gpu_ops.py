@@ -168,6 +168,37 @@ def test_expert_matches_oracle(case, device):
     assert err <= (1e-2 if dtype != torch.float32 else 1e-5) * max(scale, 1e-6), (err, scale)
 
 
+@pytest.mark.parametrize("case", EXPERT_CASES, ids=lambda c: f"T{c[0]}-H{c[1]}-N{c[2]}-k{c[3]}-{str(c[4]).split('.')[-1]}-{c[5]}")
+def test_expert_segment_algorithm_equals_gather(case, device):
+    """The expert-centric organisation (schedule -> coefficients per sorted pair -> token sum) uses
+    the same per-pair arithmetic and the same summation order: bit-identical output."""
+    T, H, N, k, dtype, kind = case
+    d = [t.to(device) for t in _expert_inputs(T, H, N, k, dtype, kind, seed=T + H)]
+    print(f"expert segment T={T} H={H} N={N} k={k} {dtype} {kind}", flush=True)
+    a = _ops().hip_omni_expert_func(*d, algo="gather")
+    b = _ops().hip_omni_expert_func(*d, algo="segment")
+    torch.cuda.synchronize()
+    assert torch.equal(a, b)
+
+
+def test_expert_segment_skewed_and_bad_ids(device):
+    g = torch.Generator().manual_seed(11)
+    T, H, N, k = 4096, 1024, 512, 8
+    x, up, down = torch.randn(T, H, generator=g).bfloat16(), (torch.randn(N, H, generator=g) * 0.05).bfloat16(), (torch.randn(N, H, generator=g) * 0.05).bfloat16()
+    gates = torch.rand(T, k, generator=g).bfloat16()
+    w = 1.0 / torch.arange(1, N + 1, dtype=torch.float64) ** 1.5            # one very hot expert
+    ids = torch.multinomial(w, T * k, replacement=True, generator=g).reshape(T, k).to(torch.int32)
+    ids[::7, 3] = N + 5                                                      # ids outside the table contribute nothing
+    ids[::11, 0] = -1
+    d = [t.to(device) for t in (x, up, down, gates, ids)]
+    a = _ops().hip_omni_expert_func(*d, algo="gather")
+    b = _ops().hip_omni_expert_func(*d, algo="segment")
+    assert torch.equal(a, b)
+    ok = (ids >= 0) & (ids < N)
+    want = oracle.expert_forward(x, up, down, torch.where(ok, gates, torch.zeros_like(gates)), torch.where(ok, ids, torch.zeros_like(ids)))
+    torch.testing.assert_close(a.cpu().float(), want.float(), rtol=2e-2, atol=2e-2)
+
+
 def test_expert_edge_cases(device):
     hip = _ops()
     x, up, down, gates, ids = (t.to(device) for t in _expert_inputs(16, 256, 32, 4, torch.bfloat16, "ref", 1))
