@@ -169,12 +169,15 @@ def main():
         x3, up3, down3, g3, i3 = (t.to(dev) for t in oracle.make_expert_inputs(2, T3, H, N, k))
         ms_e3 = time_call(torch, lambda: hip.hip_omni_expert_func(x3, up3, down3, g3, i3), reps)
         ms_s3 = time_call(torch, lambda: hip.hip_omni_schedule_func(i3, N), reps)
+        ms_seg3 = time_call(torch, lambda: hip.hip_omni_expert_func(x3, up3, down3, g3, i3, algo="segment"), reps)
         kernels.append(hbm_entry("expert_gather_kernel, c3 (T=16384)", expert_alg_bytes(T3, H, k), ms_e3,
                                  "up/down tables (16 MiB) are cache-resident, so algorithmic bytes exceed HBM traffic",
                                  TRAFFIC_BYTES["expert_c3"]))
-        kernels.append(hbm_entry("schedule (fill+histogram+scan+scatter, 5 launches), c3", T3 * k * 14 + 8 * (N + 1), ms_s3))
+        kernels.append(hbm_entry("schedule (stable counting sort: count, scan x2, scatter, offsets), c3", T3 * k * 14 + 8 * (N + 1), ms_s3))
+        kernels.append(hbm_entry("expert op, expert-centric 'segment' algorithm (schedule + scores pass + token pass), c3",
+                                 expert_alg_bytes(T3, H, k), ms_seg3, "for comparison with expert_gather_kernel; same results"))
         out["roofline"] = max(kernels[:3], key=lambda d: d["kernel_ms"])
-        out["roofline_expert"] = kernels[-2]
+        out["roofline_expert"] = kernels[-3]
         out["kernels"] = kernels
 
     if not a.no_cpu_baseline:
