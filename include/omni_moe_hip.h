@@ -129,6 +129,11 @@ OMNI_API int32_t omni_swiglu_linear_fwd(const void* x, const void* gate_weight, 
 OMNI_API int32_t omni_linear_fwd(const void* x, const void* weight, const void* residual, void* y, int64_t num_tokens,
                                  int32_t in_features, int32_t out_features, int32_t dtype, void* stream);
 
+/* y[i] = round(y[i] + addend[i]) in place: the layer's final  mlp + experts  (omni_moe.py:102) as a
+ * call of its own, for callers that run the two branches on different streams.  num_elements a
+ * multiple of 8 (4 for f32); both pointers 16-byte aligned. */
+OMNI_API int32_t omni_add_inplace(void* y, const void* addend, int64_t num_elements, int32_t dtype, void* stream);
+
 /* Two bias-free linear layers sharing their input, written side by side:
  * y[T, 2*out] = [x weight_lo^T | x weight_hi^T].  One GEMM for the router's x and y
  * projections (omni_moe.py:70-71).  out_features_each a multiple of 2. */
@@ -156,6 +161,29 @@ OMNI_API int32_t omni_router_fwd(const void* x, const void* weight_x, const void
                                  void* scores, int64_t num_tokens, int32_t hidden_size, int32_t num_expert_sqrt,
                                  int32_t num_experts_per_token, int32_t dtype, int32_t stats_dtype,
                                  void* workspace, void* stream);
+
+/* The whole layer forward in one call: replaces OmniMoE.forward (omni_moe/modules/omni_moe.py:60-106),
+ * i.e. omni_router_fwd + omni_expert_fwd + omni_mlp_fwd with the final add (:102).
+ *   x, y [T,H]; gate_weight, up_weight [I,H]; down_weight [H,I]; router_weight_x/y [r,H];
+ *   up_embed, down_embed [N,H]; BatchNorm buffers as in omni_router_fwd.
+ *   stream      : every kernel is ordered on it
+ *   side_stream : NULL, or a second stream on which the router + expert branch is enqueued while the
+ *                 MLP branch runs on `stream`; then fork_event and join_event must be two events of
+ *                 the caller (hipEvent_t, timing disabled is fine); `stream` waits for the branch before
+ *                 the final add, so after the call `stream` alone orders all later work.
+ *   workspace   : omni_moe_workspace_bytes() bytes; must stay untouched until the work has run. */
+OMNI_API size_t omni_moe_workspace_bytes(int64_t num_tokens, int32_t hidden_size, int32_t intermediate_size,
+                                         int64_t num_experts, int32_t num_expert_sqrt, int32_t num_experts_per_token,
+                                         int32_t dtype);
+OMNI_API int32_t omni_moe_fwd(const void* x, const void* gate_weight, const void* up_weight, const void* down_weight,
+                              const void* router_weight_x, const void* router_weight_y,
+                              void* running_mean_x, void* running_var_x, int64_t* num_batches_tracked_x,
+                              void* running_mean_y, void* running_var_y, int64_t* num_batches_tracked_y,
+                              const void* up_embed, const void* down_embed, void* y,
+                              int64_t num_tokens, int32_t hidden_size, int32_t intermediate_size, int64_t num_experts,
+                              int32_t num_expert_sqrt, int32_t num_experts_per_token, int32_t dtype, int32_t stats_dtype,
+                              int32_t training, float momentum, float eps, void* workspace, void* stream,
+                              void* side_stream, void* fork_event, void* join_event);
 
 #ifdef __cplusplus
 }

@@ -655,3 +655,39 @@ extern "C" OMNI_API int32_t omni_debug_set_timing(long long* buf) {
   return (int32_t)hipMemcpyToSymbol(HIP_SYMBOL(omni::g_timing), &buf, sizeof(buf));
 }
 #endif
+
+namespace omni {
+// y[i] = round(y[i] + e[i]), 8 (16-bit) or 4 (fp32) elements per lane
+template <int DT>
+__global__ __launch_bounds__(256) void add_inplace_kernel(uint8_t* __restrict__ y, const uint8_t* __restrict__ e, int64_t num_chunks) {
+  for (int64_t i = blockIdx.x * 256ll + threadIdx.x; i < num_chunks; i += gridDim.x * 256ll) {
+    const u32x4_t a = *(const u32x4_t*)(y + i * 16), b = *(const u32x4_t*)(e + i * 16);
+    u32x4_t o;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const uint32_t aq = a[q], bq = b[q];
+      if constexpr (DT == kBF16) o[q] = pack_bf16(bf16_lo(aq) + bf16_lo(bq), bf16_hi(aq) + bf16_hi(bq));
+      else if constexpr (DT == kF16) o[q] = pack_f16(f16_bits_to_f32(aq & 0xffff) + f16_bits_to_f32(bq & 0xffff), f16_bits_to_f32(aq >> 16) + f16_bits_to_f32(bq >> 16));
+      else o[q] = __float_as_uint(__uint_as_float(aq) + __uint_as_float(bq));
+    }
+    *(u32x4_t*)(y + i * 16) = o;
+  }
+}
+}  // namespace omni
+
+extern "C" OMNI_API int32_t omni_add_inplace(void* y, const void* addend, int64_t num_elements, int32_t dtype, void* stream) {
+  using namespace omni;
+  if (num_elements < 0) return OMNI_ERR_SHAPE;
+  if (dtype != OMNI_BF16 && dtype != OMNI_F16 && dtype != OMNI_F32) return OMNI_ERR_DTYPE;
+  const int per = dtype == OMNI_F32 ? 4 : 8;
+  if (num_elements % per != 0) return OMNI_ERR_SHAPE;
+  if (num_elements == 0) return OMNI_OK;
+  if (!y || !addend) return OMNI_ERR_NULL;
+  const int64_t chunks = num_elements / per;
+  const unsigned blocks = (unsigned)((chunks + 255) / 256 < 4096 ? (chunks + 255) / 256 : 4096);
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == OMNI_BF16) hipLaunchKernelGGL(add_inplace_kernel<kBF16>, dim3(blocks), dim3(256), 0, s, (uint8_t*)y, (const uint8_t*)addend, chunks);
+  else if (dtype == OMNI_F16) hipLaunchKernelGGL(add_inplace_kernel<kF16>, dim3(blocks), dim3(256), 0, s, (uint8_t*)y, (const uint8_t*)addend, chunks);
+  else hipLaunchKernelGGL(add_inplace_kernel<kF32>, dim3(blocks), dim3(256), 0, s, (uint8_t*)y, (const uint8_t*)addend, chunks);
+  return omni::to_code(hipGetLastError());
+}

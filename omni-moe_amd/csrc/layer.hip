@@ -1,0 +1,72 @@
+// The whole OmniMoE forward (reference omni_moe/modules/omni_moe.py:60-106) as one call:
+// router -> fused experts on one branch, gate/up projection -> down projection on the other,
+// joined by the final add.  With a second stream the two branches are enqueued side by side
+// (the expert kernel lives on cache bandwidth and no LDS, the down projection on LDS and the
+// matrix cores, so they share CUs); the fork and the join are two events the caller owns.
+#include "common.h"
+#include "omni_moe_hip.h"
+
+namespace omni {
+static inline size_t up256(size_t v) { return (v + 255) / 256 * 256; }
+static inline size_t elem_bytes(int dtype) { return dtype == OMNI_F32 ? 4 : 2; }
+}  // namespace omni
+
+// workspace: router workspace | gates [T,k] | ids [T,k] | expert output [T,H] | SwiGLU activations [T,I]
+extern "C" OMNI_API size_t omni_moe_workspace_bytes(int64_t num_tokens, int32_t hidden_size, int32_t intermediate_size,
+                                                    int64_t num_experts, int32_t num_expert_sqrt, int32_t num_experts_per_token,
+                                                    int32_t dtype) {
+  using namespace omni;
+  (void)num_experts;
+  if (num_tokens < 0 || hidden_size <= 0 || intermediate_size <= 0 || num_expert_sqrt <= 0 || num_experts_per_token < 0) return 0;
+  const size_t es = elem_bytes(dtype), T = (size_t)num_tokens, k = (size_t)num_experts_per_token;
+  return up256(omni_router_workspace_bytes(num_tokens, num_expert_sqrt, dtype)) + up256(T * k * es) + up256(T * k * 4) +
+         up256(T * (size_t)hidden_size * es) + up256(omni_mlp_workspace_bytes(num_tokens, hidden_size, intermediate_size, dtype));
+}
+
+extern "C" OMNI_API int32_t omni_moe_fwd(const void* x, const void* gate_weight, const void* up_weight, const void* down_weight,
+                                         const void* router_weight_x, const void* router_weight_y,
+                                         void* running_mean_x, void* running_var_x, int64_t* num_batches_tracked_x,
+                                         void* running_mean_y, void* running_var_y, int64_t* num_batches_tracked_y,
+                                         const void* up_embed, const void* down_embed, void* y,
+                                         int64_t num_tokens, int32_t hidden_size, int32_t intermediate_size, int64_t num_experts,
+                                         int32_t num_expert_sqrt, int32_t num_experts_per_token, int32_t dtype, int32_t stats_dtype,
+                                         int32_t training, float momentum, float eps, void* workspace, void* stream,
+                                         void* side_stream, void* fork_event, void* join_event) {
+  using namespace omni;
+  if (num_tokens < 0 || hidden_size <= 0 || intermediate_size <= 0 || num_experts <= 0 || num_expert_sqrt <= 0) return OMNI_ERR_SHAPE;
+  if (dtype != OMNI_BF16 && dtype != OMNI_F16 && dtype != OMNI_F32) return OMNI_ERR_DTYPE;
+  if (num_tokens == 0) return OMNI_OK;
+  if (!x || !y || !up_embed || !down_embed) return OMNI_ERR_NULL;
+  if (!workspace) return OMNI_ERR_WORKSPACE;
+  if (side_stream && (!fork_event || !join_event)) return OMNI_ERR_NULL;
+  const size_t es = elem_bytes(dtype), T = (size_t)num_tokens, k = (size_t)num_experts_per_token;
+  char* w = (char*)workspace;
+  void* router_ws = w;  w += up256(omni_router_workspace_bytes(num_tokens, num_expert_sqrt, dtype));
+  void* gates = w;      w += up256(T * k * es);
+  int32_t* ids = (int32_t*)w;  w += up256(T * k * 4);
+  void* experts = w;    w += up256(T * (size_t)hidden_size * es);
+  void* h = w;
+
+  hipStream_t main_s = (hipStream_t)stream;
+  hipStream_t branch = side_stream ? (hipStream_t)side_stream : main_s;
+  hipError_t he;
+  if (side_stream) {
+    if ((he = hipEventRecord((hipEvent_t)fork_event, main_s)) != hipSuccess) return OMNI_ERR_HIP_BASE + (int)he;
+    if ((he = hipStreamWaitEvent(branch, (hipEvent_t)fork_event, 0)) != hipSuccess) return OMNI_ERR_HIP_BASE + (int)he;
+  }
+  int e;
+  if ((e = omni_router_fwd(x, router_weight_x, router_weight_y, running_mean_x, running_var_x, num_batches_tracked_x,
+                           running_mean_y, running_var_y, num_batches_tracked_y, training, momentum, eps, gates, ids, nullptr,
+                           num_tokens, hidden_size, num_expert_sqrt, num_experts_per_token, dtype, stats_dtype, router_ws, branch)))
+    return e;
+  if ((e = omni_swiglu_linear_fwd(x, gate_weight, up_weight, h, num_tokens, hidden_size, intermediate_size, dtype, main_s))) return e;
+  if ((e = omni_expert_fwd(x, up_embed, down_embed, gates, ids, experts, num_tokens, hidden_size, num_experts,
+                           num_experts_per_token, dtype, OMNI_EXPERT_ALGO_GATHER, nullptr, branch)))
+    return e;
+  if (!side_stream)   // one stream: the add is the down projection's epilogue
+    return omni_linear_fwd(h, down_weight, experts, y, num_tokens, intermediate_size, hidden_size, dtype, main_s);
+  if ((e = omni_linear_fwd(h, down_weight, nullptr, y, num_tokens, intermediate_size, hidden_size, dtype, main_s))) return e;
+  if ((he = hipEventRecord((hipEvent_t)join_event, branch)) != hipSuccess) return OMNI_ERR_HIP_BASE + (int)he;
+  if ((he = hipStreamWaitEvent(main_s, (hipEvent_t)join_event, 0)) != hipSuccess) return OMNI_ERR_HIP_BASE + (int)he;
+  return omni_add_inplace(y, experts, (int64_t)T * hidden_size, dtype, main_s);
+}

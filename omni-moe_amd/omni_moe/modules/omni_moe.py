@@ -11,8 +11,7 @@ import math
 import torch
 import torch.nn as nn
 
-from omni_moe.ops.hip import (hip_linear_func, hip_omni_expert_func, hip_omni_mlp_func, hip_omni_router_fwd_func,
-                              hip_swiglu_linear_func)
+from omni_moe.ops.hip import hip_omni_moe_fwd_func, hip_omni_router_fwd_func
 
 
 class OmniMoEConfig:
@@ -76,38 +75,38 @@ class OmniMoE(nn.Module):
             self.top_k, training=self.training, momentum=nx.momentum, eps=nx.eps, return_scores=return_scores,
         )
 
-    # Router + experts and the gate/up projection only share their input, so they are enqueued
-    # on two HIP streams (both at the default priority) and meet again at the down projection,
-    # whose epilogue adds the expert output.  Set to False to keep everything on one stream.
+    # Router + experts and the shared MLP only share their input, so the library enqueues them on
+    # two HIP streams (both at the default priority) and joins them at the final add: the expert
+    # kernel (cache bandwidth, no LDS) shares CUs with the projections (LDS and MFMA).  Set to False
+    # to keep everything on one stream, with the add as the down projection's epilogue.
     overlap_branches = True
 
-    def _side_stream(self, device) -> "torch.cuda.Stream":
-        s = self.__dict__.get("_omni_side_stream")
-        if s is None or s.device != device:
-            s = torch.cuda.Stream(device=device)
-            self.__dict__["_omni_side_stream"] = s
-        return s
+    def _branch_resources(self, device):
+        res = self.__dict__.get("_omni_branch")
+        if res is None or res[0].device != device:
+            with torch.cuda.device(device):
+                side = torch.cuda.Stream(device=device)
+                fork, join = torch.cuda.Event(), torch.cuda.Event()
+                fork.record()                                # events come into being when first recorded
+                join.record()
+            res = (side, fork, join)
+            self.__dict__["_omni_branch"] = res
+        return res
 
     def forward(self, hidden_states: torch.Tensor, **kwargs) -> torch.Tensor:
         bsz, seq_len, _ = hidden_states.shape
+        nx, ny = self.router_norm_x, self.router_norm_y
+        if nx.momentum is None or ny.momentum is None:
+            raise NotImplementedError("cumulative-average BatchNorm (momentum=None) is not covered")
         with torch.no_grad():
             x = hidden_states.view(-1, self.hidden_size)
-            if self.overlap_branches and x.is_cuda:
-                main = torch.cuda.current_stream(x.device)
-                side = self._side_stream(x.device)
-                side.wait_stream(main)                       # x (and the weights) are ready
-                with torch.cuda.stream(side):
-                    routing_weights, indices = self.route(x)
-                    experts_states = hip_omni_expert_func(x, self.up_embed.weight, self.down_embed.weight,
-                                                          routing_weights, indices)
-                h = hip_swiglu_linear_func(x, self.gate_proj.weight, self.up_proj.weight)
-                main.wait_stream(side)
-                experts_states.record_stream(main)           # allocated on the side stream, read on this one
-                out = hip_linear_func(h, self.down_proj.weight, experts_states)
-            else:
-                routing_weights, indices = self.route(x)
-                experts_states = hip_omni_expert_func(x, self.up_embed.weight, self.down_embed.weight, routing_weights, indices)
-                # mlp + experts: the add is the down projection's epilogue
-                out = hip_omni_mlp_func(x, self.gate_proj.weight, self.up_proj.weight, self.down_proj.weight,
-                                        residual=experts_states)
+            side, fork, join = self._branch_resources(x.device) if (self.overlap_branches and x.is_cuda) else (None, None, None)
+            out = hip_omni_moe_fwd_func(
+                x, self.gate_proj.weight, self.up_proj.weight, self.down_proj.weight,
+                self.router_gate_x.weight, self.router_gate_y.weight,
+                nx.running_mean, nx.running_var, nx.num_batches_tracked,
+                ny.running_mean, ny.running_var, ny.num_batches_tracked,
+                self.up_embed.weight, self.down_embed.weight, self.top_k,
+                training=self.training, momentum=nx.momentum, eps=nx.eps,
+                side_stream=side, fork_event=fork, join_event=join)
         return out.view(bsz, seq_len, -1)

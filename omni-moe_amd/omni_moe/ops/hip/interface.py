@@ -204,6 +204,19 @@ def hip_swiglu_linear_func(x: torch.Tensor, gate_weight: torch.Tensor, up_weight
     return h
 
 
+def hip_add_inplace_func(y: torch.Tensor, addend: torch.Tensor) -> torch.Tensor:
+    """y += addend, rounded once (the layer's final ``mlp + experts``, reference omni_moe.py:102)."""
+    if y.shape != addend.shape or y.dtype != addend.dtype or y.dtype not in _lib.DTYPE_CODE:
+        raise ValueError("y and addend must match in shape and dtype (bfloat16, float16 or float32)")
+    if not (y.is_contiguous() and addend.is_contiguous()):
+        raise ValueError("y and addend must be contiguous")
+    dev = _lib.require_gpu(y, addend)
+    with torch.cuda.device(dev):
+        code = _lib.load().omni_add_inplace(_lib.ptr(y), _lib.ptr(addend), y.numel(), _lib.DTYPE_CODE[y.dtype], _lib.stream_ptr())
+    _lib.check(code, "omni_add_inplace")
+    return y
+
+
 def hip_omni_router_fwd_func(
     x: torch.Tensor,
     weight_x: torch.Tensor,
@@ -260,3 +273,53 @@ def hip_omni_router_fwd_func(
             T, H, r, k, dt, _lib.DTYPE_CODE[running_mean_x.dtype], _lib.ptr(ws), _lib.stream_ptr())
     _lib.check(code, "omni_router_fwd")
     return (gates, indices, scores) if return_scores else (gates, indices)
+
+
+def hip_omni_moe_fwd_func(
+    x: torch.Tensor,
+    gate_weight: torch.Tensor, up_weight: torch.Tensor, down_weight: torch.Tensor,
+    router_weight_x: torch.Tensor, router_weight_y: torch.Tensor,
+    running_mean_x: torch.Tensor, running_var_x: torch.Tensor, num_batches_tracked_x: Optional[torch.Tensor],
+    running_mean_y: torch.Tensor, running_var_y: torch.Tensor, num_batches_tracked_y: Optional[torch.Tensor],
+    up_embed: torch.Tensor, down_embed: torch.Tensor,
+    num_experts_per_token: int, training: bool, momentum: float = 0.1, eps: float = 1e-5,
+    side_stream: Optional["torch.cuda.Stream"] = None,
+    fork_event: Optional["torch.cuda.Event"] = None, join_event: Optional["torch.cuda.Event"] = None,
+) -> torch.Tensor:
+    """The whole layer forward (reference omni_moe.py:60-106) for ``x`` of shape (tokens, hidden) in one
+    library call.  With ``side_stream`` (and two events) the router + expert branch is enqueued next
+    to the MLP branch; the current stream waits for it before the final add."""
+    T, H = x.shape
+    I, N, r, k = gate_weight.size(0), up_embed.size(0), router_weight_x.size(0), int(num_experts_per_token)
+    weights = (gate_weight, up_weight, down_weight, router_weight_x, router_weight_y, up_embed, down_embed)
+    if x.dim() != 2 or x.dtype not in _lib.DTYPE_CODE or any(t.dtype != x.dtype or not t.is_contiguous() for t in weights):
+        raise TypeError("x and the weights must be contiguous and share a dtype in {bfloat16, float16, float32}")
+    if (gate_weight.shape != (I, H) or up_weight.shape != (I, H) or down_weight.shape != (H, I) or router_weight_y.shape != (r, H)
+            or router_weight_x.shape != (r, H) or up_embed.shape != (N, H) or down_embed.shape != (N, H)):
+        raise ValueError("weight shapes do not fit (tokens, hidden) input")
+    stats = (running_mean_x, running_var_x, running_mean_y, running_var_y)
+    if any(t.dtype != running_mean_x.dtype or t.shape != (r,) or not t.is_contiguous() for t in stats) or running_mean_x.dtype not in _lib.DTYPE_CODE:
+        raise ValueError("running statistics must be contiguous (num_expert_sqrt,) tensors of one floating dtype")
+    assert 0 <= k <= r * r, f"num_experts_per_token should be in [0, {r * r}], but got {k}"
+    assert k <= 128, "num_experts_per_token should be less than or equal to 128"
+    assert k % 2 == 0, "num_experts_per_token should be a multiple of 2"
+    dev = _lib.require_gpu(x, *weights, *stats)
+    x = _c(x)
+    lib = _lib.load()
+    dt = _lib.DTYPE_CODE[x.dtype]
+    y = torch.empty_like(x)
+    ws = torch.empty(max(lib.omni_moe_workspace_bytes(T, H, I, N, r, k, dt), 1), device=dev, dtype=torch.uint8)
+    side = fork = join = 0
+    if side_stream is not None:
+        side, fork, join = side_stream.cuda_stream, fork_event.cuda_event, join_event.cuda_event
+    with torch.cuda.device(dev):
+        code = lib.omni_moe_fwd(
+            _lib.ptr(x), _lib.ptr(gate_weight), _lib.ptr(up_weight), _lib.ptr(down_weight), _lib.ptr(router_weight_x),
+            _lib.ptr(router_weight_y), _lib.ptr(running_mean_x), _lib.ptr(running_var_x), _lib.ptr(num_batches_tracked_x),
+            _lib.ptr(running_mean_y), _lib.ptr(running_var_y), _lib.ptr(num_batches_tracked_y), _lib.ptr(up_embed),
+            _lib.ptr(down_embed), _lib.ptr(y), T, H, I, N, r, k, dt, _lib.DTYPE_CODE[running_mean_x.dtype],
+            1 if training else 0, float(momentum), float(eps), _lib.ptr(ws), _lib.stream_ptr(), side, fork, join)
+    _lib.check(code, "omni_moe_fwd")
+    # ws is released here: the current stream has been made to wait for the side branch, so every
+    # later use of that memory (allocated from this stream's pool) is ordered after both branches
+    return y
