@@ -255,3 +255,36 @@ def test_layer_config5_large_skewed(device):
     assert set_agree >= 0.999
     torch.testing.assert_close(y.view(-1, H)[sub.to(device)].float().cpu(), want.view(-1, H).float(), rtol=2e-2, atol=2e-2)
     torch.testing.assert_close(gates.cpu()[sub].float(), want_g.float(), rtol=2e-2, atol=2e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=["bf16", "f32"])
+def test_layer_two_streams_equals_one_stream(dtype, device):
+    """The two-stream schedule (router+experts beside the MLP, joined by omni_add_inplace) and the
+    one-stream schedule (add fused into the down projection) give bit-identical output, call after call."""
+    from omni_moe.modules.omni_moe import OmniMoE, OmniMoEConfig
+    torch.manual_seed(0)
+    layer = OmniMoE(OmniMoEConfig(256, 512, "silu", 1024, 8)).to(device=device, dtype=dtype).eval()
+    x = torch.randn(3, 100, 256, device=device).to(dtype)
+    layer.overlap_branches = False
+    ref = layer(x)
+    layer.overlap_branches = True
+    for _ in range(5):
+        assert torch.equal(layer(x), ref)
+    # and next to other work on the caller's stream
+    s = torch.cuda.Stream()
+    with torch.cuda.stream(s):
+        z = x * 2
+        out = layer(z)
+    s.synchronize()
+    layer.overlap_branches = False
+    assert torch.equal(out, layer(x * 2))
+
+
+def test_add_inplace(device):
+    hip = _ops()
+    for dtype in (torch.bfloat16, torch.float16, torch.float32):
+        a, b = torch.randn(37, 64, device=device).to(dtype), torch.randn(37, 64, device=device).to(dtype)
+        want = (a.float() + b.float()).to(dtype)
+        assert torch.equal(hip.hip_add_inplace_func(a.clone(), b), want)
+    with pytest.raises(ValueError):
+        hip.hip_add_inplace_func(torch.zeros(4, 8, device=device), torch.zeros(4, 9, device=device))
