@@ -31,7 +31,7 @@ constexpr int kBK = 64;                       // K elements per LDS stage
 constexpr int kRowBytes = kBK * 2 + 16;       // padded LDS row
 constexpr int kGemmThreads = 256;
 
-enum : int { kEpiPlain = 0, kEpiSwiglu = 1, kEpiResidual = 2 };
+enum : int { kEpiPlain = 0, kEpiSwiglu = 1, kEpiResidual = 2, kEpiStats = 3 };   // kEpiStats: plain + column statistics
 
 template <int DT> struct ElemBytes { static constexpr int value = (DT == kF32) ? 4 : 2; };
 
@@ -70,7 +70,7 @@ struct GemmArgs {           // all element offsets below are scaled by the eleme
   int M, N, K;            // N = output columns
   int tiles_m, tiles_n;
   int patch_m, patch_n;   // XCD patch shape (0 = plain order)
-  float* part_mean;       // plain epilogue only, may be NULL: [ceil(M/32)][N] mean of each column over
+  float* part_mean;       // kEpiStats only: [ceil(M/32)][N] mean of each column over
   float* part_m2;         //   rows 32s..32s+31 of the ROUNDED result, and the sum of squared deviations
 };
 
@@ -99,7 +99,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, f32x16_t (&acc)
   constexpr int TNO = (EPI == kEpiSwiglu) ? TN / 2 : TN;
   // ---- column statistics of the rounded tile for BatchNorm: every 32-row MFMA tile is one
   // strip; a column lives in the 32 lanes that share lane/32, so five xor-shuffles reduce it
-  if constexpr (EPI == kEpiPlain) {
+  if constexpr (EPI == kEpiStats) {
     if (g.part_mean) {
 #pragma unroll
       for (int i = 0; i < TM; ++i) {
@@ -227,7 +227,7 @@ __global__ __launch_bounds__(kGemmThreads, 1) void gemm_nt_kernel(const GemmArgs
       col = n0 + p * 32 + ld_row;
     }
     col = col < g.N ? col : g.N - 1;
-    if constexpr (EPI == kEpiPlain) {
+    if constexpr (EPI == kEpiPlain || EPI == kEpiStats) {
       // optional second weight matrix supplies the upper half of the output columns
       if (g.b1 && col >= g.N / 2) { base = g.b1; col -= g.N / 2; }
     }
@@ -357,7 +357,7 @@ __global__ __launch_bounds__(kGemmThreads, 1) void gemm_nt_dma_kernel(const Gemm
       col = n0 + rl;
     }
     col = col < g.N ? col : g.N - 1;
-    if constexpr (EPI == kEpiPlain) {
+    if constexpr (EPI == kEpiPlain || EPI == kEpiStats) {
       if (g.b1 && col >= g.N / 2) { base = g.b1; col -= g.N / 2; }
     }
     b_src[p] = base + ((int64_t)col * g.K + c * 8) * 2;
@@ -542,6 +542,10 @@ static int gemm_plain(const void* a, const void* b, const void* b_hi, const void
     if (big >= 200) err = launch_gemm<DT, 4, 4, kEpiResidual>(g, s);
     else if (mid >= 200) err = launch_gemm<DT, 2, 2, kEpiResidual>(g, s);
     else err = launch_gemm<DT, 1, 1, kEpiResidual>(g, s);
+  } else if (part_mean) {
+    // the statistics keep every accumulator live through a long reduction: 128 x 128 tiles at most
+    if (mid >= 200) err = launch_gemm<DT, 2, 2, kEpiStats>(g, s);
+    else err = launch_gemm<DT, 1, 1, kEpiStats>(g, s);
   } else {
     if (big >= 200) err = launch_gemm<DT, 4, 4, kEpiPlain>(g, s);
     else if (mid >= 200) err = launch_gemm<DT, 2, 2, kEpiPlain>(g, s);

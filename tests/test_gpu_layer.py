@@ -288,3 +288,27 @@ def test_add_inplace(device):
         assert torch.equal(hip.hip_add_inplace_func(a.clone(), b), want)
     with pytest.raises(ValueError):
         hip.hip_add_inplace_func(torch.zeros(4, 8, device=device), torch.zeros(4, 9, device=device))
+
+
+# (M, N, K) that select the 128 x 128 output tiles (too few 256 x 256 tiles to fill the chip), ragged M included
+LINEAR_CASES = [(3300, 1024, 512), (3300, 1024, 640), (3300, 1024, 576), (4096, 1024, 4096), (2049, 1536, 1024)]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+@pytest.mark.parametrize("case", LINEAR_CASES, ids=lambda c: f"M{c[0]}-N{c[1]}-K{c[2]}")
+def test_linear_mid_tiles(case, dtype, device):
+    """y = x W^T (+ residual) on the 128 x 128 tile path, ragged M included, against an fp64 matmul."""
+    M, N, K = case
+    g = torch.Generator().manual_seed(M + K)
+    x = torch.randn(M, K, generator=g).to(dtype)
+    w = (torch.randn(N, K, generator=g) * 0.05).to(dtype)
+    res = torch.randn(M, N, generator=g).to(dtype)
+    print(f"linear M={M} N={N} K={K} {dtype}", flush=True)
+    want = x.double() @ w.double().t()
+    got = _ops().hip_linear_func(x.to(device), w.to(device)).cpu()
+    # one rounding of an fp32 sum: half an ulp of the storage dtype plus fp32 summation noise
+    ulp = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
+    err = (got.double() - want).abs()
+    assert (err <= ulp * want.abs() * 1.01 + 1e-4 * want.abs().max()).all()
+    got_r = _ops().hip_linear_func(x.to(device), w.to(device), residual=res.to(device)).cpu()
+    assert torch.equal(got_r, (got.float() + res.float()).to(dtype))
