@@ -18,7 +18,7 @@ namespace omni {
 
 #ifdef OMNI_GEMM_TIMING
 __device__ long long* g_timing = nullptr;   // [blocks][8] cycle stamps, debug builds only
-#define OMNI_STAMP(slot) do { if (g_timing && threadIdx.x == 0) g_timing[blockIdx.x * 8 + (slot)] = (long long)__builtin_readcyclecounter(); } while (0)
+#define OMNI_STAMP(slot) do { if (g_timing && threadIdx.x == 0) { g_timing[blockIdx.x * 8 + (slot)] = (long long)__builtin_readcyclecounter(); g_timing[blockIdx.x * 8 + 4 + (slot)] = (long long)wall_clock64(); } } while (0)
 #else
 #define OMNI_STAMP(slot) do { } while (0)
 #endif
@@ -70,6 +70,7 @@ struct GemmArgs {           // all element offsets below are scaled by the eleme
   int M, N, K;            // N = output columns
   int tiles_m, tiles_n;
   int patch_m, patch_n;   // XCD patch shape (0 = plain order)
+  int wide;               // 16-bit output: N % 8 == 0 and C 16-byte aligned, rows are written 16 bytes per lane
   float* part_mean;       // kEpiStats only: [ceil(M/32)][N] mean of each column over
   float* part_m2;         //   rows 32s..32s+31 of the ROUNDED result, and the sum of squared deviations
 };
@@ -130,29 +131,71 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, f32x16_t (&acc)
   }
 
   // ---- epilogue.  acc[i][j][q]: row m = lane%32, column n = (q/4)*8 + (lane/32)*4 + q%4
+  // value q of column group q4 after the element-wise tail, not yet rounded to storage
+  auto value = [&](int i, int j, int q4, int q) -> float {
+    if constexpr (EPI == kEpiSwiglu) {
+      // the reference materialises gate and up in the storage dtype, then forms
+      // silu(gate)*up in fp32 and rounds once (omni_mlp.py:53-61)
+      const float gt = Elem<DT>::round(acc[i][j][q4 * 4 + q]);
+      const float up = Elem<DT>::round(acc[i][j + TNO][q4 * 4 + q]);
+      return (DT == kF32) ? silu_f32(gt) * up : silu_fast(gt) * up;
+    } else {
+      return acc[i][j][q4 * 4 + q];
+    }
+  };
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
     const int m = m0 + wm * TM * 32 + i * 32 + (lane & 31);
     if (m >= g.M) continue;
 #pragma unroll
     for (int j = 0; j < TNO; ++j) {
+      const int nt = n0 + wn * TNO * 32 + j * 32;
+      if constexpr (DT != kF32) {
+        if (g.wide) {
+          // lanes l and l+32 hold columns 8*q4+{0..3} and 8*q4+{4..7} of the same row: one
+          // v_permlane32_swap per word regroups two column groups into 8 consecutive columns per
+          // lane, so a row receives full 32-byte sectors from every store instruction
+#pragma unroll
+          for (int pr = 0; pr < 2; ++pr) {
+            if (nt + pr * 16 >= g.N) continue;             // same answer in both lanes of a pair
+            uint32_t w[2][2];
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+              const int q4 = 2 * pr + e;
+              float v[4];
+#pragma unroll
+              for (int q = 0; q < 4; ++q) v[q] = value(i, j, q4, q);
+              if constexpr (EPI == kEpiResidual) {
+                const int n = nt + q4 * 8 + (lane >> 5) * 4;
+                u32x2_t r = {0u, 0u};                      // columns past N are exchanged but never stored
+                if (n < g.N) r = *(const u32x2_t*)(g.res + ((int64_t)m * g.N + n) * 2);
+                const uint32_t r0 = r[0], r1 = r[1];
+                if constexpr (DT == kBF16) {
+                  v[0] = Elem<DT>::round(v[0]) + bf16_lo(r0); v[1] = Elem<DT>::round(v[1]) + bf16_hi(r0);
+                  v[2] = Elem<DT>::round(v[2]) + bf16_lo(r1); v[3] = Elem<DT>::round(v[3]) + bf16_hi(r1);
+                } else {
+                  v[0] = Elem<DT>::round(v[0]) + f16_bits_to_f32(r0 & 0xffff); v[1] = Elem<DT>::round(v[1]) + f16_bits_to_f32(r0 >> 16);
+                  v[2] = Elem<DT>::round(v[2]) + f16_bits_to_f32(r1 & 0xffff); v[3] = Elem<DT>::round(v[3]) + f16_bits_to_f32(r1 >> 16);
+                }
+              }
+              w[e][0] = pack2<DT>(v[0], v[1]);
+              w[e][1] = pack2<DT>(v[2], v[3]);
+            }
+            const auto s0 = __builtin_amdgcn_permlane32_swap(w[0][0], w[1][0], false, false);
+            const auto s1 = __builtin_amdgcn_permlane32_swap(w[0][1], w[1][1], false, false);
+            const int n = nt + pr * 16 + (lane >> 5) * 8;
+            if (n < g.N) *(u32x4_t*)(g.c + ((int64_t)m * g.N + n) * 2) = u32x4_t{s0[0], s1[0], s0[1], s1[1]};
+          }
+          continue;
+        }
+      }
 #pragma unroll
       for (int q4 = 0; q4 < 4; ++q4) {
-        const int n = n0 + wn * TNO * 32 + j * 32 + q4 * 8 + (lane >> 5) * 4;
+        const int n = nt + q4 * 8 + (lane >> 5) * 4;
         if (n >= g.N) continue;                          // N is a multiple of 4
         float v[4];
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          if constexpr (EPI == kEpiSwiglu) {
-            // the reference materialises gate and up in the storage dtype, then forms
-            // silu(gate)*up in fp32 and rounds once (omni_mlp.py:53-61)
-            const float gt = Elem<DT>::round(acc[i][j][q4 * 4 + q]);
-            const float up = Elem<DT>::round(acc[i][j + TNO][q4 * 4 + q]);
-            v[q] = (DT == kF32) ? silu_f32(gt) * up : silu_fast(gt) * up;
-          } else {
-            v[q] = acc[i][j][q4 * 4 + q];
-          }
-        }
+        for (int q = 0; q < 4; ++q) v[q] = value(i, j, q4, q);
         const int64_t o = ((int64_t)m * g.N + n) * ElemBytes<DT>::value;
         if constexpr (EPI == kEpiResidual) {
           // y = round(h Wd^T) + e, rounded again: the reference adds two stored tensors
@@ -486,6 +529,7 @@ static hipError_t launch_gemm(GemmArgs g, hipStream_t s) {
   const int blocks = g.tiles_m * g.tiles_n;
   // one XCD runs 32 blocks at a time: give it 4 x 8 patches when the tile grid allows
   g.patch_m = g.patch_n = 0;
+  g.wide = (DT != kF32) && g.N % 8 == 0 && ((uintptr_t)g.c % 16 == 0);
   if (blocks % 256 == 0) {
     if (g.tiles_m % 4 == 0 && g.tiles_n % 8 == 0) { g.patch_m = 4; g.patch_n = 8; }
     else if (g.tiles_m % 8 == 0 && g.tiles_n % 4 == 0) { g.patch_m = 8; g.patch_n = 4; }
@@ -533,7 +577,7 @@ static int gemm_plain(const void* a, const void* b, const void* b_hi, const void
                       float* part_mean = nullptr, float* part_m2 = nullptr) {
   if (int e = check_gemm(M, N, K, ElemBytes<DT>::value)) return e;
   if (M == 0) return OMNI_OK;
-  GemmArgs g{(const uint8_t*)a, (const uint8_t*)b, (const uint8_t*)b_hi, (const uint8_t*)res, (uint8_t*)c, (int)M, (int)N, (int)K, 0, 0, 0, 0, nullptr, nullptr};
+  GemmArgs g{(const uint8_t*)a, (const uint8_t*)b, (const uint8_t*)b_hi, (const uint8_t*)res, (uint8_t*)c, (int)M, (int)N, (int)K, 0, 0, 0, 0, 0, nullptr, nullptr};
   g.part_mean = part_mean;
   g.part_m2 = part_m2;
   const int64_t big = ((M + 255) / 256) * ((N + 255) / 256), mid = ((M + 127) / 128) * ((N + 127) / 128);
@@ -558,7 +602,7 @@ template <int DT>
 static int gemm_swiglu(const void* x, const void* wg, const void* wu, void* h, int64_t M, int64_t I, int64_t K, hipStream_t s) {
   if (int e = check_gemm(M, I, K, ElemBytes<DT>::value)) return e;
   if (M == 0) return OMNI_OK;
-  GemmArgs g{(const uint8_t*)x, (const uint8_t*)wg, (const uint8_t*)wu, nullptr, (uint8_t*)h, (int)M, (int)I, (int)K, 0, 0, 0, 0, nullptr, nullptr};
+  GemmArgs g{(const uint8_t*)x, (const uint8_t*)wg, (const uint8_t*)wu, nullptr, (uint8_t*)h, (int)M, (int)I, (int)K, 0, 0, 0, 0, 0, nullptr, nullptr};
   const int64_t big = ((M + 255) / 256) * ((I + 127) / 128);
   hipError_t err;
   if (big >= 200) err = launch_gemm<DT, 4, 4, kEpiSwiglu>(g, s);

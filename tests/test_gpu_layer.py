@@ -290,14 +290,16 @@ def test_add_inplace(device):
         hip.hip_add_inplace_func(torch.zeros(4, 8, device=device), torch.zeros(4, 9, device=device))
 
 
-# (M, N, K) that select the 128 x 128 output tiles (too few 256 x 256 tiles to fill the chip), ragged M included
-LINEAR_CASES = [(3300, 1024, 512), (3300, 1024, 640), (3300, 1024, 576), (4096, 1024, 4096), (2049, 1536, 1024)]
+# (M, N, K): the first five select the 128 x 128 output tiles (too few 256 x 256 tiles to fill the chip), ragged M
+# included; then a big-tile case, N % 8 == 4 (rows written 8 bytes per lane instead of 16) and a ragged last column tile
+LINEAR_CASES = [(3300, 1024, 512), (3300, 1024, 640), (3300, 1024, 576), (4096, 1024, 4096), (2049, 1536, 1024),
+                (4096, 4096, 256), (300, 100, 264), (333, 1000, 256), (70, 4, 8)]
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
 @pytest.mark.parametrize("case", LINEAR_CASES, ids=lambda c: f"M{c[0]}-N{c[1]}-K{c[2]}")
-def test_linear_mid_tiles(case, dtype, device):
-    """y = x W^T (+ residual) on the 128 x 128 tile path, ragged M included, against an fp64 matmul."""
+def test_linear_matches_matmul(case, dtype, device):
+    """y = x W^T (+ residual) against an fp64 matmul, over the tile shapes and both store widths."""
     M, N, K = case
     g = torch.Generator().manual_seed(M + K)
     x = torch.randn(M, K, generator=g).to(dtype)
