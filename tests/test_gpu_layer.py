@@ -314,3 +314,30 @@ def test_linear_matches_matmul(case, dtype, device):
     assert (err <= ulp * want.abs() * 1.01 + 1e-4 * want.abs().max()).all()
     got_r = _ops().hip_linear_func(x.to(device), w.to(device), residual=res.to(device)).cpu()
     assert torch.equal(got_r, (got.float() + res.float()).to(dtype))
+
+
+@pytest.mark.parametrize("overlap", [True, False], ids=["two-streams", "one-stream"])
+def test_layer_is_graph_capturable(overlap, device):
+    """The library only launches kernels and records/waits events, so a whole layer forward (fork and join
+    included) can be captured into a HIP graph; every replay, with eager work in between, equals the eager result."""
+    from omni_moe.modules.omni_moe import OmniMoE, OmniMoEConfig
+    torch.manual_seed(1)
+    layer = OmniMoE(OmniMoEConfig(256, 512, "silu", 1024, 8)).to(device=device, dtype=torch.bfloat16).eval()
+    layer.overlap_branches = overlap
+    x = torch.randn(2, 150, 256, device=device).bfloat16()
+    want = layer(x).clone()
+    warm = torch.cuda.Stream()
+    warm.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(warm):
+        layer(x)
+    torch.cuda.current_stream().wait_stream(warm)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        y = layer(x)
+    for _ in range(4):
+        y.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y, want)
+        assert torch.equal(layer(x * 0.5), layer(x * 0.5))      # eager work between the replays
+        torch.cuda.synchronize()
