@@ -161,7 +161,7 @@ def main():
             mfma_entry("gemm_nt_dma_kernel<residual> (down projection + experts add), c4", 2 * T * H * I, ms_down, TRAFFIC_BYTES["down_c4"]),
             hbm_entry("expert_gather_kernel, c4", expert_alg_bytes(T, H, k), ms_expert,
                       "up/down tables (16 MiB) are cache-resident, so algorithmic bytes exceed HBM traffic", TRAFFIC_BYTES["expert_c4"]),
-            {"kernel": "router stage (linear2 GEMM + BN partial + BN finalize + select), c4", "kernel_ms": ms_router,
+            {"kernel": "router stage (projection GEMM with BN statistics epilogue + BN finalize + select), c4", "kernel_ms": ms_router,
              "algorithmic_flops": 4 * T * H * r},
         ]
         # expert kernel at the shape its bandwidth target is quoted on (BASELINE config 3)

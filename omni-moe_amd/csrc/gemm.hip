@@ -6,11 +6,11 @@
 //   * down projection     y  = h Wd^T (+ expert output)        (interface.py:23-29, omni_moe.py:102)
 //
 // Structure: a block of 4 waves (2 x 2) owns a (2*TM*32) x (2*TN*32) tile; each wave owns
-// TM x TN MFMA tiles of 32x32.  K advances 64 at a time: global 128-bit loads go to
-// registers, then into one of two LDS stages whose rows are padded by 16 bytes so that the
-// 128-bit fragment reads of 16 consecutive rows hit all 64 banks once.  The weight fragment
-// is the MFMA's first operand, so an accumulator lane holds 4 consecutive output columns of
-// one row and stores them as one 8-byte word.
+// TM x TN MFMA tiles of 32x32 and K advances 64 at a time.  16-bit operands with K % 64 == 0
+// take `gemm_nt_dma_kernel` (global -> LDS directly, ring of stages, swizzled rows); anything
+// else takes `gemm_nt_kernel` (global -> registers -> one of two LDS stages with padded rows).
+// The weight fragment is the MFMA's first operand, so an accumulator lane holds 4 consecutive
+// output columns of one row; two lanes pair up to store 8 columns (16 bytes) each.
 #include "common.h"
 #include "omni_moe_hip.h"
 

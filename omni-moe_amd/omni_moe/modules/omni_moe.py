@@ -1,10 +1,12 @@
 """OmniMoE layer: drop-in for the reference's ``omni_moe.modules.omni_moe`` (forward path).
 
 Same constructor, attribute / ``state_dict`` names and ``forward(hidden_states, **kwargs)``
-as the reference's ``OmniMoE`` (omni_moe/modules/omni_moe.py:14-106); the forward runs three
-calls into the gfx950 library: router (projection, BatchNorm, log-softmax, Cartesian top-k,
-exp), fused atomic experts, and the shared SwiGLU MLP whose down projection adds the expert
-output.  Forward only: outputs carry no autograd graph.
+as the reference's ``OmniMoE`` (omni_moe/modules/omni_moe.py:14-106); the forward is ONE call
+into the gfx950 library (``omni_moe_fwd``): router (projection, BatchNorm, log-softmax,
+Cartesian top-k, exp) and fused experts on a side stream, the shared SwiGLU MLP on the
+caller's stream, joined by the final add (``overlap_branches = False``: everything on the
+caller's stream, the add fused into the down projection).  Forward only: outputs carry no
+autograd graph.
 """
 import math
 
