@@ -90,6 +90,7 @@ def main():
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    torch.set_grad_enabled(False)          # forward path: the module then issues its single fused library call
 
     # ---------------- BASELINE config 4: README-shape full layer
     T, H, I, N, k, seed = 4096, 1024, 4096, 4096, 16, 3

@@ -134,6 +134,47 @@ OMNI_API int32_t omni_linear_fwd(const void* x, const void* weight, const void* 
  * multiple of 8 (4 for f32); both pointers 16-byte aligned. */
 OMNI_API int32_t omni_add_inplace(void* y, const void* addend, int64_t num_elements, int32_t dtype, void* stream);
 
+/* ---- backward of the three operators (the training path) ----------------------------------- */
+
+/* Router backward: the gradient of the selected scores scatters to the two half-logit rows,
+ * dlogits_x[t, ix] += dscores[t, j], dlogits_y[t, iy] += dscores[t, j] for id = ix*r + iy.
+ * Replaces _omni_router_backward (omni_moe/ops/triton/omni_router.py:235-274, kernel :98-164).
+ *   dscores [T,k] dtype `dtype`; indices [T,k] int32 as returned by omni_router_select (ids outside
+ *   [0, r*r) are skipped); dlogits_x, dlogits_y [T,r] dtype `dtype`, fully overwritten.
+ * fp32 sums in slot order (the reference uses fp32 atomics), one rounding.  r <= 1024, k <= 128. */
+OMNI_API int32_t omni_router_bwd(const void* dscores, const int32_t* indices, void* dlogits_x, void* dlogits_y,
+                                 int64_t num_tokens, int32_t num_expert_sqrt, int32_t num_experts_per_token,
+                                 int32_t dtype, void* stream);
+
+/* Fused atomic-expert backward.  For pair (t, e = indices[t,j]) with s = <x_t, U_e>, a = <dy_t, V_e>,
+ * g = routing_weights[t,j]:  drouting_weights[t,j] = a silu(s);  dx_t += a g silu'(s) U_e;
+ * dup_weight[e] += a g silu'(s) x_t;  ddown_weight[e] += silu(s) g dy_t.
+ * Replaces omni_expert_backward (omni_expert.py:1067-1277, kernels :375-618).  s is recomputed (the
+ * forward saves nothing); every output is fully overwritten (rows of experts nobody selected are
+ * zero); sums are fp32 in a fixed order with one rounding, no atomics.
+ *   dy, x, dx [T,H]; up_weight, down_weight, dup_weight, ddown_weight [N,H]; routing_weights,
+ *   drouting_weights [T,k] : dtype `dtype`; indices [T,k] int32 (ids outside [0,N) contribute nothing)
+ *   workspace : omni_expert_bwd_workspace_bytes() bytes */
+OMNI_API size_t omni_expert_bwd_workspace_bytes(int64_t num_tokens, int32_t hidden_size, int64_t num_experts,
+                                                int32_t num_experts_per_token, int32_t dtype);
+OMNI_API int32_t omni_expert_bwd(const void* dy, const void* x, const void* up_weight, const void* down_weight,
+                                 const void* routing_weights, const int32_t* indices, void* dx, void* dup_weight,
+                                 void* ddown_weight, void* drouting_weights, int64_t num_tokens, int32_t hidden_size,
+                                 int64_t num_experts, int32_t num_experts_per_token, int32_t dtype, void* workspace,
+                                 void* stream);
+
+/* Element-wise SwiGLU for the training path, which keeps gate and up:
+ *   omni_swiglu_fwd: out = silu(gate) * up, fp32 product, one rounding
+ *                    (TritonSwiGLUFunc.forward, omni_mlp.py:252-303, kernel :102-177, math :53-61)
+ *   omni_swiglu_bwd: dup = dout * silu(gate);  dgate = dout * (silu(gate) (1 - sig) + sig) * up
+ *                    (TritonSwiGLUFunc.backward, omni_mlp.py:306-356, kernel :180-249)
+ * num_elements a multiple of 8 (4 for f32); pointers 16-byte aligned. */
+OMNI_API int32_t omni_swiglu_fwd(const void* gate, const void* up, void* out, int64_t num_elements, int32_t dtype,
+                                 void* stream);
+OMNI_API int32_t omni_swiglu_bwd(const void* dout, const void* gate, const void* up, void* dgate, void* dup,
+                                 int64_t num_elements, int32_t dtype, void* stream);
+
+
 /* Two bias-free linear layers sharing their input, written side by side:
  * y[T, 2*out] = [x weight_lo^T | x weight_hi^T].  One GEMM for the router's x and y
  * projections (omni_moe.py:70-71).  out_features_each a multiple of 2. */

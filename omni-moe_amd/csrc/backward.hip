@@ -1,0 +1,402 @@
+// Backward kernels of the three OmniMoE operators for gfx950, so that a layer built on them
+// trains.  Each replaces the matching Triton backward of the reference:
+//   * router   (omni_moe/ops/triton/omni_router.py:98-164, 235-274): the gradient of the k
+//     selected scores scatters back to the two half-logit rows, d_lx[ix] += ds, d_ly[iy] += ds;
+//   * experts  (omni_expert.py:375-618, 1067-1277): for a pair (t, e) with s = <x_t, U_e>,
+//     a = <dy_t, V_e>:   dg = a silu(s),   ds = a g silu'(s),   dx_t += ds U_e,
+//     dU_e += ds x_t,   dV_e += silu(s) g dy_t;
+//   * SwiGLU   (omni_mlp.py:102-177 forward, 180-249 backward) as element-wise kernels for
+//     the training path, which keeps gate and up (the inference path forms the product in the
+//     GEMM epilogue and never stores them).
+// All sums are fp32 in a fixed order, rounded once on the way out: no atomics anywhere (the
+// reference accumulates dx, dU and dV with atomics in the storage dtype), so gradients are
+// run-to-run identical.
+//
+// Expert backward in two passes.  Token pass: one wave owns one token, keeps x_t, dy_t and the
+// fp32 dx accumulator in registers, fetches each selected up and down row once, recomputes s
+// (nothing is saved by the forward), writes dg and, to an fp32 workspace, ds and the forward
+// coefficient silu(s) g of every pair.  Weight pass: the pairs are grouped by expert with the
+// stable schedule of the forward path; one wave owns one expert, walks its segment and gathers
+// the x and dy rows of the segment's tokens, so every dU/dV row is written exactly once
+// (zeros for experts nobody selected).
+#include "common.h"
+#include "omni_moe_hip.h"
+#include "rows.h"
+
+namespace omni {
+
+constexpr int kBwdWavesPerBlock = 4;
+
+__device__ __forceinline__ float sigmoid_f32(float x) { return 1.0f / (1.0f + __expf(-x)); }
+
+// ---- router ------------------------------------------------------------------------------------
+// One wave per token; lane l accumulates columns l, l+64, ... of both halves (r <= 1024).
+template <int DT>
+__global__ __launch_bounds__(kBwdWavesPerBlock* kWave) void router_bwd_kernel(
+    const void* __restrict__ dscores, const int32_t* __restrict__ ids, void* __restrict__ dlx, void* __restrict__ dly,
+    int num_tokens, int r, int top_k) {
+  constexpr int kCols = 16;                         // 16 * 64 = 1024 columns per half
+  const int lane = lane_id();
+  const int t = __builtin_amdgcn_readfirstlane(blockIdx.x * kBwdWavesPerBlock + (threadIdx.x >> 6));
+  if (t >= num_tokens) return;
+  float ax[kCols], ay[kCols];
+#pragma unroll
+  for (int c = 0; c < kCols; ++c) ax[c] = ay[c] = 0.f;
+  const int64_t base = int64_t(t) * top_k;
+  for (int j0 = 0; j0 < top_k; j0 += kWave) {       // k <= 128: at most two rounds
+    const int j = j0 + lane;
+    const int my_id = j < top_k ? ids[base + j] : -1;
+    const float my_ds = j < top_k ? Elem<DT>::load(dscores, base + j) : 0.f;
+    const int n = min(kWave, top_k - j0);
+    for (int i = 0; i < n; ++i) {                   // slot order: the sum per column is deterministic
+      const int id = __shfl(my_id, i, kWave);
+      const float ds = __shfl(my_ds, i, kWave);
+      if ((uint32_t)id >= (uint32_t)r * (uint32_t)r) continue;   // uniform: an id outside the product is ignored
+      const int ix = id / r, iy = id - ix * r;
+#pragma unroll
+      for (int c = 0; c < kCols; ++c) {
+        ax[c] += (ix == c * kWave + lane) ? ds : 0.f;
+        ay[c] += (iy == c * kWave + lane) ? ds : 0.f;
+      }
+    }
+  }
+#pragma unroll
+  for (int c = 0; c < kCols; ++c) {
+    const int col = c * kWave + lane;
+    if (col < r) {
+      Elem<DT>::store(dlx, int64_t(t) * r + col, ax[c]);
+      Elem<DT>::store(dly, int64_t(t) * r + col, ay[c]);
+    }
+  }
+}
+
+// ---- experts, token pass -----------------------------------------------------------------------
+template <int DT, int NCH, int G>
+__global__ __launch_bounds__(kBwdWavesPerBlock* kWave, 2) void expert_bwd_token_kernel(
+    const uint8_t* __restrict__ x, const uint8_t* __restrict__ dy, const uint8_t* __restrict__ up,
+    const uint8_t* __restrict__ down, const void* __restrict__ gates, const int32_t* __restrict__ ids,
+    uint8_t* __restrict__ dx, void* __restrict__ dgates, float* __restrict__ ds_out, float* __restrict__ coef_out,
+    int num_tokens, int hidden, int top_k, uint32_t num_experts) {
+  constexpr int E = Row16<DT>::kElems;
+  const int lane = lane_id();
+  const int t = __builtin_amdgcn_readfirstlane(blockIdx.x * kBwdWavesPerBlock + (threadIdx.x >> 6));
+  if (t >= num_tokens) return;
+  const int64_t row_bytes = int64_t(hidden) * (16 / E);
+
+  bool live[NCH];
+  int64_t off[NCH];
+  u32x4_t xr[NCH], dyr[NCH];
+  float acc[NCH][E];
+#pragma unroll
+  for (int c = 0; c < NCH; ++c) {
+    live[c] = (c * kWave + lane) * E < hidden;
+    off[c] = int64_t(c * kWave + lane) * 16;
+    xr[c] = live[c] ? *(const u32x4_t*)(x + t * row_bytes + off[c]) : u32x4_t{0, 0, 0, 0};
+    dyr[c] = live[c] ? *(const u32x4_t*)(dy + t * row_bytes + off[c]) : u32x4_t{0, 0, 0, 0};
+#pragma unroll
+    for (int i = 0; i < E; ++i) acc[c][i] = 0.f;
+  }
+
+  const int64_t base = int64_t(t) * top_k;
+  for (int j0 = 0; j0 < top_k; j0 += G) {
+    int e[G];
+    float g[G];
+    bool live_slot[G];
+#pragma unroll
+    for (int i = 0; i < G; ++i) {
+      const int j = min(j0 + i, top_k - 1);
+      const int id = ids[base + j];
+      const float gate = Elem<DT>::load(gates, base + j);
+      const bool ok = (j0 + i < top_k) && (uint32_t)id < num_experts;   // as the forward: such a pair contributes nothing
+      e[i] = ok ? id : 0;
+      g[i] = ok ? gate : 0.f;
+      live_slot[i] = ok;
+    }
+    u32x4_t ur[G][NCH], vr[G][NCH];
+#pragma unroll
+    for (int i = 0; i < G; ++i)
+#pragma unroll
+      for (int c = 0; c < NCH; ++c)
+        ur[i][c] = live[c] ? *(const u32x4_t*)(up + e[i] * row_bytes + off[c]) : u32x4_t{0, 0, 0, 0};
+#pragma unroll
+    for (int i = 0; i < G; ++i)
+#pragma unroll
+      for (int c = 0; c < NCH; ++c)
+        vr[i][c] = live[c] ? *(const u32x4_t*)(down + e[i] * row_bytes + off[c]) : u32x4_t{0, 0, 0, 0};
+
+    float s[G], a[G];
+#pragma unroll
+    for (int i = 0; i < G; ++i) {
+      float ps = 0.f, pa = 0.f;
+#pragma unroll
+      for (int c = 0; c < NCH; ++c) {
+        ps = dot16<DT>(xr[c], ur[i][c], ps);
+        pa = dot16<DT>(dyr[c], vr[i][c], pa);
+      }
+      s[i] = ps;
+      a[i] = pa;
+    }
+#pragma unroll
+    for (int i = 0; i < G; ++i) {
+      s[i] = wave_sum(s[i]);
+      a[i] = wave_sum(a[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < G; ++i) {
+      const float sig = sigmoid_f32(s[i]);
+      const float silu = s[i] * sig;
+      const float dsilu = sig + silu * (1.0f - sig);
+      const float dg = live_slot[i] ? a[i] * silu : 0.f;
+      const float ds = live_slot[i] ? a[i] * g[i] * dsilu : 0.f;
+      const float coef = live_slot[i] ? silu * g[i] : 0.f;
+      if (lane == 0 && j0 + i < top_k) {
+        Elem<DT>::store(dgates, base + j0 + i, dg);
+        ds_out[base + j0 + i] = ds;
+        coef_out[base + j0 + i] = coef;
+      }
+#pragma unroll
+      for (int c = 0; c < NCH; ++c) axpy16<DT>(ds, ur[i][c], acc[c]);
+    }
+  }
+#pragma unroll
+  for (int c = 0; c < NCH; ++c)
+    if (live[c]) *(u32x4_t*)(dx + t * row_bytes + off[c]) = pack16<DT>(acc[c]);
+}
+
+// ---- experts, weight pass ----------------------------------------------------------------------
+template <int DT, int NCH, int G>
+__global__ __launch_bounds__(kBwdWavesPerBlock* kWave, 2) void expert_bwd_weight_kernel(
+    const uint8_t* __restrict__ x, const uint8_t* __restrict__ dy, const float* __restrict__ ds, const float* __restrict__ coef,
+    const int32_t* __restrict__ offsets, const int32_t* __restrict__ sorted_pair_ids, const int32_t* __restrict__ sorted_token_ids,
+    uint8_t* __restrict__ dup, uint8_t* __restrict__ ddown, int64_t num_experts, int hidden) {
+  constexpr int E = Row16<DT>::kElems;
+  const int lane = lane_id();
+  const int64_t e = __builtin_amdgcn_readfirstlane((int)(blockIdx.x * kBwdWavesPerBlock + (threadIdx.x >> 6)));
+  if (e >= num_experts) return;
+  const int64_t row_bytes = int64_t(hidden) * (16 / E);
+  const int begin = offsets[e], end = offsets[e + 1];
+
+  bool live[NCH];
+  int64_t off[NCH];
+  float au[NCH][E], av[NCH][E];
+#pragma unroll
+  for (int c = 0; c < NCH; ++c) {
+    live[c] = (c * kWave + lane) * E < hidden;
+    off[c] = int64_t(c * kWave + lane) * 16;
+#pragma unroll
+    for (int i = 0; i < E; ++i) au[c][i] = av[c][i] = 0.f;
+  }
+  for (int p0 = begin; p0 < end; p0 += G) {          // segment order = pair order: a fixed summation order
+    int64_t tok[G];
+    float cs[G], cc[G];
+#pragma unroll
+    for (int i = 0; i < G; ++i) {
+      const int p = min(p0 + i, end - 1);
+      const int pid = sorted_pair_ids[p];
+      tok[i] = sorted_token_ids[p];
+      const bool ok = p0 + i < end;
+      cs[i] = ok ? ds[pid] : 0.f;
+      cc[i] = ok ? coef[pid] : 0.f;
+    }
+    u32x4_t xr[G][NCH], dyr[G][NCH];
+#pragma unroll
+    for (int i = 0; i < G; ++i)
+#pragma unroll
+      for (int c = 0; c < NCH; ++c) {
+        xr[i][c] = live[c] ? *(const u32x4_t*)(x + tok[i] * row_bytes + off[c]) : u32x4_t{0, 0, 0, 0};
+        dyr[i][c] = live[c] ? *(const u32x4_t*)(dy + tok[i] * row_bytes + off[c]) : u32x4_t{0, 0, 0, 0};
+      }
+#pragma unroll
+    for (int i = 0; i < G; ++i)
+#pragma unroll
+      for (int c = 0; c < NCH; ++c) {
+        axpy16<DT>(cs[i], xr[i][c], au[c]);
+        axpy16<DT>(cc[i], dyr[i][c], av[c]);
+      }
+  }
+#pragma unroll
+  for (int c = 0; c < NCH; ++c)
+    if (live[c]) {
+      *(u32x4_t*)(dup + e * row_bytes + off[c]) = pack16<DT>(au[c]);
+      *(u32x4_t*)(ddown + e * row_bytes + off[c]) = pack16<DT>(av[c]);
+    }
+}
+
+// ---- SwiGLU, element-wise ----------------------------------------------------------------------
+// 16 bytes per lane.  Forward: out = silu(gate) * up in fp32, one rounding (omni_mlp.py:53-61).
+// Backward: with a = gate in fp32, sig = sigmoid(a):  d_up = dout * a sig,
+// d_gate = dout * (a sig (1 - sig) + sig) * up  (omni_mlp.py:232-236).
+template <int DT, bool BWD>
+__global__ __launch_bounds__(256) void swiglu_kernel(const uint8_t* __restrict__ dout, const uint8_t* __restrict__ gate,
+                                                    const uint8_t* __restrict__ up, uint8_t* __restrict__ out0,
+                                                    uint8_t* __restrict__ out1, int64_t num_chunks) {
+  constexpr int E = Row16<DT>::kElems;
+  for (int64_t i = blockIdx.x * 256ll + threadIdx.x; i < num_chunks; i += gridDim.x * 256ll) {
+    const u32x4_t gw = *(const u32x4_t*)(gate + i * 16), uw = *(const u32x4_t*)(up + i * 16);
+    float gv[E], uv[E], r0[E], r1[E];
+    unpack16<DT>(gw, gv);
+    unpack16<DT>(uw, uv);
+    if constexpr (BWD) {
+      float dv[E];
+      unpack16<DT>(*(const u32x4_t*)(dout + i * 16), dv);
+#pragma unroll
+      for (int q = 0; q < E; ++q) {
+        const float sig = sigmoid_f32(gv[q]), silu = gv[q] * sig;
+        r0[q] = dv[q] * (silu * (1.0f - sig) + sig) * uv[q];
+        r1[q] = dv[q] * silu;
+      }
+      *(u32x4_t*)(out0 + i * 16) = pack16<DT>(r0);
+      *(u32x4_t*)(out1 + i * 16) = pack16<DT>(r1);
+    } else {
+#pragma unroll
+      for (int q = 0; q < E; ++q) r0[q] = gv[q] * sigmoid_f32(gv[q]) * uv[q];
+      *(u32x4_t*)(out0 + i * 16) = pack16<DT>(r0);
+    }
+  }
+}
+
+// ---- host side ---------------------------------------------------------------------------------
+static inline size_t up256(size_t v) { return (v + 255) / 256 * 256; }
+static int to_code(hipError_t e) { return e == hipSuccess ? OMNI_OK : OMNI_ERR_HIP_BASE + (int)e; }
+
+template <int DT, int NCH, int G>
+static hipError_t launch_expert_bwd(const void* dy, const void* x, const void* up, const void* down, const void* gates,
+                                    const int32_t* ids, void* dx, void* dup, void* ddown, void* dgates, float* ds, float* coef,
+                                    const int32_t* offsets, const int32_t* pair_ids, const int32_t* token_ids, int64_t T, int H,
+                                    int64_t N, int k, hipStream_t s) {
+  dim3 block(kBwdWavesPerBlock * kWave);
+  if (T > 0) {
+    dim3 grid((unsigned)((T + kBwdWavesPerBlock - 1) / kBwdWavesPerBlock));
+    hipLaunchKernelGGL((expert_bwd_token_kernel<DT, NCH, G>), grid, block, 0, s, (const uint8_t*)x, (const uint8_t*)dy,
+                       (const uint8_t*)up, (const uint8_t*)down, gates, ids, (uint8_t*)dx, dgates, ds, coef, (int)T, H, k,
+                       (uint32_t)N);
+    if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
+  }
+  dim3 grid((unsigned)((N + kBwdWavesPerBlock - 1) / kBwdWavesPerBlock));
+  hipLaunchKernelGGL((expert_bwd_weight_kernel<DT, NCH, G>), grid, block, 0, s, (const uint8_t*)x, (const uint8_t*)dy, ds, coef,
+                     offsets, pair_ids, token_ids, (uint8_t*)dup, (uint8_t*)ddown, N, H);
+  return hipGetLastError();
+}
+
+}  // namespace omni
+
+extern "C" OMNI_API int32_t omni_router_bwd(const void* dscores, const int32_t* indices, void* dlogits_x, void* dlogits_y,
+                                            int64_t num_tokens, int32_t num_expert_sqrt, int32_t num_experts_per_token,
+                                            int32_t dtype, void* stream) {
+  using namespace omni;
+  if (num_tokens < 0 || num_tokens > INT32_MAX || num_expert_sqrt <= 0 || num_experts_per_token < 0) return OMNI_ERR_SHAPE;
+  if (num_expert_sqrt > 1024) return OMNI_ERR_UNSUPPORTED;
+  if (num_experts_per_token > 128) return OMNI_ERR_TOPK;
+  if (dtype != OMNI_BF16 && dtype != OMNI_F16 && dtype != OMNI_F32) return OMNI_ERR_DTYPE;
+  if (num_tokens == 0) return OMNI_OK;
+  if (!dlogits_x || !dlogits_y || (num_experts_per_token > 0 && (!dscores || !indices))) return OMNI_ERR_NULL;
+  dim3 grid((unsigned)((num_tokens + kBwdWavesPerBlock - 1) / kBwdWavesPerBlock)), block(kBwdWavesPerBlock * kWave);
+  hipStream_t s = (hipStream_t)stream;
+  const int T = (int)num_tokens, r = num_expert_sqrt, k = num_experts_per_token;
+  if (dtype == OMNI_BF16) hipLaunchKernelGGL(router_bwd_kernel<kBF16>, grid, block, 0, s, dscores, indices, dlogits_x, dlogits_y, T, r, k);
+  else if (dtype == OMNI_F16) hipLaunchKernelGGL(router_bwd_kernel<kF16>, grid, block, 0, s, dscores, indices, dlogits_x, dlogits_y, T, r, k);
+  else hipLaunchKernelGGL(router_bwd_kernel<kF32>, grid, block, 0, s, dscores, indices, dlogits_x, dlogits_y, T, r, k);
+  return to_code(hipGetLastError());
+}
+
+// workspace: ds [P] f32 | coef [P] f32 | offsets [N+1] i32 | sorted pair ids [P] i32 | sorted token ids [P] i32 | schedule workspace
+extern "C" OMNI_API size_t omni_expert_bwd_workspace_bytes(int64_t num_tokens, int32_t hidden_size, int64_t num_experts,
+                                                           int32_t num_experts_per_token, int32_t dtype) {
+  using namespace omni;
+  (void)hidden_size;
+  (void)dtype;
+  if (num_tokens < 0 || num_experts <= 0 || num_experts_per_token < 0) return 0;
+  const size_t P = (size_t)num_tokens * (size_t)num_experts_per_token;
+  return 4 * up256(P * 4) + up256(((size_t)num_experts + 1) * 4) +
+         omni_schedule_workspace_bytes(num_tokens, num_experts_per_token, num_experts);
+}
+
+extern "C" OMNI_API int32_t omni_expert_bwd(const void* dy, const void* x, const void* up_weight, const void* down_weight,
+                                            const void* routing_weights, const int32_t* indices, void* dx, void* dup_weight,
+                                            void* ddown_weight, void* drouting_weights, int64_t num_tokens, int32_t hidden_size,
+                                            int64_t num_experts, int32_t num_experts_per_token, int32_t dtype, void* workspace,
+                                            void* stream) {
+  using namespace omni;
+  if (num_tokens < 0 || hidden_size <= 0 || num_experts <= 0 || num_experts_per_token < 0) return OMNI_ERR_SHAPE;
+  if (num_tokens > INT32_MAX / 2 || num_experts > INT32_MAX / 2 ||
+      num_tokens * (int64_t)num_experts_per_token > INT32_MAX / 2)
+    return OMNI_ERR_SHAPE;
+  if (dtype != OMNI_BF16 && dtype != OMNI_F16 && dtype != OMNI_F32) return OMNI_ERR_DTYPE;
+  if (!dup_weight || !ddown_weight) return OMNI_ERR_NULL;
+  if (num_tokens > 0 && (!dy || !x || !dx || !up_weight || !down_weight)) return OMNI_ERR_NULL;
+  if (num_tokens > 0 && num_experts_per_token > 0 && (!routing_weights || !indices || !drouting_weights)) return OMNI_ERR_NULL;
+  if (!workspace) return OMNI_ERR_WORKSPACE;
+  const int E = dtype == OMNI_F32 ? 4 : 8;
+  if (hidden_size % E != 0) return OMNI_ERR_SHAPE;
+  const int nch = (hidden_size + kWave * E - 1) / (kWave * E);
+  if (nch > 8) return OMNI_ERR_UNSUPPORTED;
+  const size_t P = (size_t)num_tokens * (size_t)num_experts_per_token;
+  char* w = (char*)workspace;
+  float* ds = (float*)w;               w += up256(P * 4);
+  float* coef = (float*)w;             w += up256(P * 4);
+  int32_t* pair_ids = (int32_t*)w;     w += up256(P * 4);
+  int32_t* token_ids = (int32_t*)w;    w += up256(P * 4);
+  int32_t* offsets = (int32_t*)w;      w += up256(((size_t)num_experts + 1) * 4);
+  hipStream_t s = (hipStream_t)stream;
+  if (int e = omni_schedule(indices, offsets, pair_ids, token_ids, num_tokens, num_experts_per_token, num_experts, w, stream)) return e;
+  const int64_t T = num_tokens, N = num_experts;
+  const int H = hidden_size, k = num_experts_per_token;
+  hipError_t err;
+#define OMNI_BWD_CASE(DT)                                                                                                         \
+  do {                                                                                                                            \
+    if (nch <= 1) err = launch_expert_bwd<DT, 1, 8>(dy, x, up_weight, down_weight, routing_weights, indices, dx, dup_weight,     \
+                                                    ddown_weight, drouting_weights, ds, coef, offsets, pair_ids, token_ids, T,   \
+                                                    H, N, k, s);                                                                  \
+    else if (nch <= 2) err = launch_expert_bwd<DT, 2, 8>(dy, x, up_weight, down_weight, routing_weights, indices, dx,            \
+                                                         dup_weight, ddown_weight, drouting_weights, ds, coef, offsets,          \
+                                                         pair_ids, token_ids, T, H, N, k, s);                                    \
+    else if (nch <= 4) err = launch_expert_bwd<DT, 4, 4>(dy, x, up_weight, down_weight, routing_weights, indices, dx,            \
+                                                         dup_weight, ddown_weight, drouting_weights, ds, coef, offsets,          \
+                                                         pair_ids, token_ids, T, H, N, k, s);                                    \
+    else err = launch_expert_bwd<DT, 8, 2>(dy, x, up_weight, down_weight, routing_weights, indices, dx, dup_weight,              \
+                                           ddown_weight, drouting_weights, ds, coef, offsets, pair_ids, token_ids, T, H, N, k,   \
+                                           s);                                                                                    \
+  } while (0)
+  if (dtype == OMNI_BF16) OMNI_BWD_CASE(kBF16);
+  else if (dtype == OMNI_F16) OMNI_BWD_CASE(kF16);
+  else OMNI_BWD_CASE(kF32);
+#undef OMNI_BWD_CASE
+  return to_code(err);
+}
+
+static int32_t swiglu_launch(bool bwd, const void* dout, const void* gate, const void* up, void* out0, void* out1,
+                             int64_t num_elements, int32_t dtype, void* stream) {
+  using namespace omni;
+  if (num_elements < 0) return OMNI_ERR_SHAPE;
+  if (dtype != OMNI_BF16 && dtype != OMNI_F16 && dtype != OMNI_F32) return OMNI_ERR_DTYPE;
+  const int E = dtype == OMNI_F32 ? 4 : 8;
+  if (num_elements % E != 0) return OMNI_ERR_SHAPE;
+  if (num_elements == 0) return OMNI_OK;
+  if (!gate || !up || !out0 || (bwd && (!dout || !out1))) return OMNI_ERR_NULL;
+  const int64_t chunks = num_elements / E;
+  const int64_t want = (chunks + 255) / 256;
+  dim3 grid((unsigned)(want < 8192 ? want : 8192)), block(256);
+  hipStream_t s = (hipStream_t)stream;
+  const uint8_t *d = (const uint8_t*)dout, *g = (const uint8_t*)gate, *u = (const uint8_t*)up;
+  uint8_t *o0 = (uint8_t*)out0, *o1 = (uint8_t*)out1;
+#define OMNI_SWIGLU_CASE(DT)                                                                            \
+  do {                                                                                                  \
+    if (bwd) hipLaunchKernelGGL((swiglu_kernel<DT, true>), grid, block, 0, s, d, g, u, o0, o1, chunks); \
+    else hipLaunchKernelGGL((swiglu_kernel<DT, false>), grid, block, 0, s, d, g, u, o0, o1, chunks);    \
+  } while (0)
+  if (dtype == OMNI_BF16) OMNI_SWIGLU_CASE(kBF16);
+  else if (dtype == OMNI_F16) OMNI_SWIGLU_CASE(kF16);
+  else OMNI_SWIGLU_CASE(kF32);
+#undef OMNI_SWIGLU_CASE
+  return to_code(hipGetLastError());
+}
+
+extern "C" OMNI_API int32_t omni_swiglu_fwd(const void* gate, const void* up, void* out, int64_t num_elements, int32_t dtype,
+                                            void* stream) {
+  return swiglu_launch(false, nullptr, gate, up, out, nullptr, num_elements, dtype, stream);
+}
+
+extern "C" OMNI_API int32_t omni_swiglu_bwd(const void* dout, const void* gate, const void* up, void* dgate, void* dup,
+                                            int64_t num_elements, int32_t dtype, void* stream) {
+  return swiglu_launch(true, dout, gate, up, dgate, dup, num_elements, dtype, stream);
+}

@@ -43,6 +43,11 @@ SIGNATURES = {
     "omni_router_fwd": (c_int32, [c_void_p] * 9 + [c_int32, c_float, c_float, c_void_p, c_void_p, c_void_p,
                                   c_int64, c_int32, c_int32, c_int32, c_int32, c_int32, c_void_p, c_void_p]),
     "omni_expert_fwd": (c_int32, [c_void_p] * 6 + [c_int64, c_int32, c_int64, c_int32, c_int32, c_int32, c_void_p, c_void_p]),
+    "omni_router_bwd": (c_int32, [c_void_p] * 4 + [c_int64, c_int32, c_int32, c_int32, c_void_p]),
+    "omni_expert_bwd_workspace_bytes": (c_size_t, [c_int64, c_int32, c_int64, c_int32, c_int32]),
+    "omni_expert_bwd": (c_int32, [c_void_p] * 10 + [c_int64, c_int32, c_int64, c_int32, c_int32, c_void_p, c_void_p]),
+    "omni_swiglu_fwd": (c_int32, [c_void_p] * 3 + [c_int64, c_int32, c_void_p]),
+    "omni_swiglu_bwd": (c_int32, [c_void_p] * 5 + [c_int64, c_int32, c_void_p]),
 }
 
 _lib = None

@@ -18,7 +18,7 @@ INCLUDE = os.path.join(REPO_ROOT, "include")
 LIB_PATH = os.path.join(HERE, "libomni_moe_hip.so")
 OBJ_DIR = os.path.join(PKG_ROOT, "build")
 
-SOURCES = ["api.hip", "router.hip", "schedule.hip", "expert.hip", "gemm.hip", "layer.hip"]
+SOURCES = ["api.hip", "router.hip", "schedule.hip", "expert.hip", "gemm.hip", "layer.hip", "backward.hip"]
 
 # packed-fp32 VALU forms are switched off for all device code of this library
 HIPCC_FLAGS = [

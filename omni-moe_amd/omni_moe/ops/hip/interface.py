@@ -3,7 +3,11 @@
 Same call signatures, shapes, dtypes and return arity as the reference's
 ``omni_moe/ops/triton/interface.py`` (router :32-51, expert :54-72, mlp :7-29); the
 work is done by hand-written gfx950 kernels behind the C ABI in
-``include/omni_moe_hip.h``.  Forward only.
+``include/omni_moe_hip.h``.  Like the reference's operators they are differentiable: when
+autograd is recording and an input requires grad, the router, expert and MLP operators go
+through ``torch.autograd.Function`` wrappers (``OmniRouterFunc``, ``OmniExpertFunc``,
+``OmniSwiGLUFunc``, ``OmniLinearFunc``) whose backward passes are HIP kernels too (GEMM
+gradients are library matmuls, as in the reference).  Otherwise no graph is built.
 """
 from __future__ import annotations
 
@@ -42,9 +46,19 @@ def hip_omni_router_func(
         raise ValueError("router logits must have num_expert_sqrt columns")
     if router_logits_x.dtype != router_logits_y.dtype or router_logits_x.dtype not in _lib.DTYPE_CODE:
         raise TypeError("router logits must share a dtype in {bfloat16, float16, float32}")
-    dev = _lib.require_gpu(router_logits_x, router_logits_y)
-    lx, ly = _c(router_logits_x), _c(router_logits_y)
-    T = lx.size(0)
+    _lib.require_gpu(router_logits_x, router_logits_y)
+    if _needs_grad(router_logits_x, router_logits_y):
+        return OmniRouterFunc.apply(router_logits_x, router_logits_y, r, k)
+    return _router_select(router_logits_x, router_logits_y, r, k)
+
+
+def _needs_grad(*tensors) -> bool:
+    return torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors)
+
+
+def _router_select(lx: torch.Tensor, ly: torch.Tensor, r: int, k: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    lx, ly = _c(lx.detach()), _c(ly.detach())
+    dev, T = lx.device, lx.size(0)
     scores = torch.empty((T, k), device=dev, dtype=lx.dtype)
     indices = torch.empty((T, k), device=dev, dtype=torch.int32)
     with torch.cuda.device(dev):
@@ -53,6 +67,44 @@ def hip_omni_router_func(
             _lib.DTYPE_CODE[lx.dtype], _lib.stream_ptr())
     _lib.check(code, "omni_router_select")
     return scores, indices
+
+
+def hip_omni_router_bwd_func(dscores: torch.Tensor, indices: torch.Tensor, num_expert_sqrt: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Gradient of the selected scores w.r.t. the two half-logit tensors, each [T, r] in dscores' dtype
+    (``_omni_router_backward``, reference omni_router.py:235-274)."""
+    if dscores.dim() != 2 or dscores.shape != indices.shape or indices.dtype != torch.int32:
+        raise ValueError("dscores and int32 indices must both be (num_tokens, num_experts_per_token)")
+    if dscores.dtype not in _lib.DTYPE_CODE:
+        raise TypeError("dscores must be bfloat16, float16 or float32")
+    dev = _lib.require_gpu(dscores, indices)
+    dscores, indices = _c(dscores), _c(indices)
+    T, k = dscores.shape
+    r = int(num_expert_sqrt)
+    dlx = torch.empty((T, r), device=dev, dtype=dscores.dtype)
+    dly = torch.empty((T, r), device=dev, dtype=dscores.dtype)
+    with torch.cuda.device(dev):
+        code = _lib.load().omni_router_bwd(_lib.ptr(dscores), _lib.ptr(indices), _lib.ptr(dlx), _lib.ptr(dly), T, r, k,
+                                           _lib.DTYPE_CODE[dscores.dtype], _lib.stream_ptr())
+    _lib.check(code, "omni_router_bwd")
+    return dlx, dly
+
+
+class OmniRouterFunc(torch.autograd.Function):
+    """Differentiable Cartesian top-k (mirrors ``OmniRouterFunc``, reference omni_router.py:277-307)."""
+
+    @staticmethod
+    def forward(ctx, router_logits_x, router_logits_y, num_expert_sqrt, num_experts_per_token):
+        scores, indices = _router_select(router_logits_x, router_logits_y, num_expert_sqrt, num_experts_per_token)
+        ctx.save_for_backward(indices)
+        ctx.num_expert_sqrt = num_expert_sqrt
+        ctx.mark_non_differentiable(indices)
+        return scores, indices
+
+    @staticmethod
+    def backward(ctx, dscores, _dindices):
+        (indices,) = ctx.saved_tensors
+        dlx, dly = hip_omni_router_bwd_func(dscores, indices, ctx.num_expert_sqrt)
+        return dlx, dly, None, None
 
 
 class Schedule(NamedTuple):
@@ -112,8 +164,18 @@ def hip_omni_expert_func(
         raise TypeError("x, up_weight, down_weight, routing_weights must share a dtype in {bfloat16, float16, float32}")
     if indices.dtype != torch.int32:
         indices = indices.to(torch.int32)
-    dev = _lib.require_gpu(x, up_weight, down_weight, routing_weights, indices)
-    x, up_weight, down_weight, routing_weights, indices = map(_c, (x, up_weight, down_weight, routing_weights, indices))
+    _lib.require_gpu(x, up_weight, down_weight, routing_weights, indices)
+    if _needs_grad(x, up_weight, down_weight, routing_weights):
+        if algo not in ("auto", "gather"):
+            raise ValueError("the differentiable expert op uses the default algorithm")
+        return OmniExpertFunc.apply(x, up_weight, down_weight, routing_weights, indices)
+    return _expert_forward(x, up_weight, down_weight, routing_weights, indices, algo)
+
+
+def _expert_forward(x, up_weight, down_weight, routing_weights, indices, algo="auto"):
+    x, up_weight, down_weight, routing_weights, indices = (
+        _c(t.detach()) for t in (x, up_weight, down_weight, routing_weights, indices))
+    dev = x.device
     T, H = x.shape
     N, k = up_weight.size(0), indices.size(1)
     lib = _lib.load()
@@ -126,6 +188,44 @@ def hip_omni_expert_func(
                                    _lib.ptr(indices), _lib.ptr(y), T, H, N, k, dt, al, _lib.ptr(ws), _lib.stream_ptr())
     _lib.check(code, "omni_expert_fwd")
     return y
+
+
+def hip_omni_expert_bwd_func(dy, x, up_weight, down_weight, routing_weights, indices):
+    """Gradients of the expert op: (dx [T,H], dup_weight [N,H], ddown_weight [N,H], drouting_weights [T,k]),
+    each in the dtype of its primal (``omni_expert_backward``, reference omni_expert.py:1067-1277)."""
+    if dy.shape != x.shape or dy.dtype != x.dtype:
+        raise ValueError("dy must match x in shape and dtype")
+    dev = _lib.require_gpu(dy, x, up_weight, down_weight, routing_weights, indices)
+    dy, x, up_weight, down_weight, routing_weights, indices = map(_c, (dy, x, up_weight, down_weight, routing_weights, indices))
+    T, H = x.shape
+    N, k = up_weight.size(0), indices.size(1)
+    lib = _lib.load()
+    dt = _lib.DTYPE_CODE[x.dtype]
+    dx, dup, ddown, dg = torch.empty_like(x), torch.empty_like(up_weight), torch.empty_like(down_weight), torch.empty_like(routing_weights)
+    ws = torch.empty(max(lib.omni_expert_bwd_workspace_bytes(T, H, N, k, dt), 1), device=dev, dtype=torch.uint8)
+    with torch.cuda.device(dev):
+        code = lib.omni_expert_bwd(_lib.ptr(dy), _lib.ptr(x), _lib.ptr(up_weight), _lib.ptr(down_weight), _lib.ptr(routing_weights),
+                                   _lib.ptr(indices), _lib.ptr(dx), _lib.ptr(dup), _lib.ptr(ddown), _lib.ptr(dg), T, H, N, k, dt,
+                                   _lib.ptr(ws), _lib.stream_ptr())
+    _lib.check(code, "omni_expert_bwd")
+    return dx, dup, ddown, dg
+
+
+class OmniExpertFunc(torch.autograd.Function):
+    """Differentiable fused expert op (mirrors ``OmniExpertFunc``, reference omni_expert.py:1280-1360).
+    Only the inputs are saved: the backward recomputes the pair scores."""
+
+    @staticmethod
+    def forward(ctx, x, up_weight, down_weight, routing_weights, indices):
+        y = _expert_forward(x, up_weight, down_weight, routing_weights, indices)
+        ctx.save_for_backward(x, up_weight, down_weight, routing_weights, indices)
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, up_weight, down_weight, routing_weights, indices = ctx.saved_tensors
+        dx, dup, ddown, dg = hip_omni_expert_bwd_func(dy, x, up_weight, down_weight, routing_weights, indices)
+        return dx, dup, ddown, dg, None
 
 
 def hip_omni_mlp_func(
@@ -155,8 +255,14 @@ def hip_omni_mlp_func(
             raise ValueError("residual must match x in shape and dtype")
         tensors.append(residual)
     dev = _lib.require_gpu(*tensors)
-    x, gate_weight, up_weight, down_weight = map(_c, (x, gate_weight, up_weight, down_weight))
-    residual = _c(residual) if residual is not None else None
+    if _needs_grad(*tensors):
+        # the reference's composition (interface.py:23-29): three matmuls around the SwiGLU function
+        gate = OmniLinearFunc.apply(x, gate_weight)
+        up = OmniLinearFunc.apply(x, up_weight)
+        y = OmniLinearFunc.apply(OmniSwiGLUFunc.apply(gate, up), down_weight)
+        return y if residual is None else y + residual
+    x, gate_weight, up_weight, down_weight = (_c(t.detach()) for t in (x, gate_weight, up_weight, down_weight))
+    residual = _c(residual.detach()) if residual is not None else None
     lib = _lib.load()
     dt = _lib.DTYPE_CODE[x.dtype]
     y = torch.empty_like(x)
@@ -176,15 +282,88 @@ def hip_linear_func(x: torch.Tensor, weight: torch.Tensor, residual: Optional[to
         raise TypeError("x and weight must share a dtype in {bfloat16, float16, float32}")
     if residual is not None and (residual.shape != (x.size(0), weight.size(0)) or residual.dtype != x.dtype):
         raise ValueError("residual must be (tokens, out) in x's dtype")
-    dev = _lib.require_gpu(x, weight)
-    x, weight = _c(x), _c(weight)
-    residual = _c(residual) if residual is not None else None
+    _lib.require_gpu(x, weight)
+    if _needs_grad(x, weight, residual):
+        y = OmniLinearFunc.apply(x, weight)
+        return y if residual is None else y + residual
+    return _linear_forward(x, weight, residual)
+
+
+def _linear_forward(x, weight, residual=None):
+    x, weight = _c(x.detach()), _c(weight.detach())
+    residual = _c(residual.detach()) if residual is not None else None
+    dev = x.device
     y = torch.empty((x.size(0), weight.size(0)), device=dev, dtype=x.dtype)
     with torch.cuda.device(dev):
         code = _lib.load().omni_linear_fwd(_lib.ptr(x), _lib.ptr(weight), _lib.ptr(residual), _lib.ptr(y), x.size(0), x.size(1),
                                            weight.size(0), _lib.DTYPE_CODE[x.dtype], _lib.stream_ptr())
     _lib.check(code, "omni_linear_fwd")
     return y
+
+
+class OmniLinearFunc(torch.autograd.Function):
+    """y = x W^T with the forward on the gfx950 GEMM; the two gradient GEMMs are library matmuls, as the
+    reference's ``torch.matmul`` calls get from autograd (interface.py:23-29)."""
+
+    @staticmethod
+    def forward(ctx, x, weight):
+        ctx.save_for_backward(x, weight)
+        return _linear_forward(x, weight)
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, weight = ctx.saved_tensors
+        dx = dy.matmul(weight) if ctx.needs_input_grad[0] else None
+        dw = dy.t().matmul(x) if ctx.needs_input_grad[1] else None
+        return dx, dw
+
+
+def hip_swiglu_func(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+    """silu(gate) * up element-wise, fp32 inside, one rounding (``TritonSwiGLUFunc``, reference omni_mlp.py:359-371)."""
+    if gate.shape != up.shape or gate.dtype != up.dtype or gate.dtype not in _lib.DTYPE_CODE:
+        raise ValueError("gate and up must match in shape and dtype (bfloat16, float16 or float32)")
+    _lib.require_gpu(gate, up)
+    if _needs_grad(gate, up):
+        return OmniSwiGLUFunc.apply(gate, up)
+    return _swiglu_forward(gate, up)
+
+
+def _swiglu_forward(gate, up):
+    gate, up = _c(gate.detach()), _c(up.detach())
+    out = torch.empty_like(gate)
+    with torch.cuda.device(gate.device):
+        code = _lib.load().omni_swiglu_fwd(_lib.ptr(gate), _lib.ptr(up), _lib.ptr(out), gate.numel(),
+                                           _lib.DTYPE_CODE[gate.dtype], _lib.stream_ptr())
+    _lib.check(code, "omni_swiglu_fwd")
+    return out
+
+
+def hip_swiglu_bwd_func(dout, gate, up):
+    """(dgate, dup) of ``hip_swiglu_func`` (reference omni_mlp.py:306-356)."""
+    if dout.shape != gate.shape or gate.shape != up.shape or len({dout.dtype, gate.dtype, up.dtype}) != 1:
+        raise ValueError("dout, gate and up must match in shape and dtype")
+    _lib.require_gpu(dout, gate, up)
+    dout, gate, up = _c(dout), _c(gate), _c(up)
+    dgate, dup = torch.empty_like(gate), torch.empty_like(up)
+    with torch.cuda.device(gate.device):
+        code = _lib.load().omni_swiglu_bwd(_lib.ptr(dout), _lib.ptr(gate), _lib.ptr(up), _lib.ptr(dgate), _lib.ptr(dup),
+                                           gate.numel(), _lib.DTYPE_CODE[gate.dtype], _lib.stream_ptr())
+    _lib.check(code, "omni_swiglu_bwd")
+    return dgate, dup
+
+
+class OmniSwiGLUFunc(torch.autograd.Function):
+    """Differentiable element-wise SwiGLU (mirrors ``TritonSwiGLUFunc``, reference omni_mlp.py:359-371)."""
+
+    @staticmethod
+    def forward(ctx, gate, up):
+        ctx.save_for_backward(gate, up)
+        return _swiglu_forward(gate, up)
+
+    @staticmethod
+    def backward(ctx, dout):
+        gate, up = ctx.saved_tensors
+        return hip_swiglu_bwd_func(dout, gate, up)
 
 
 def hip_swiglu_linear_func(x: torch.Tensor, gate_weight: torch.Tensor, up_weight: torch.Tensor) -> torch.Tensor:

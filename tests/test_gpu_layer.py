@@ -7,6 +7,14 @@ from oracle import omni_oracle as oracle
 pytestmark = pytest.mark.gpu
 
 
+@pytest.fixture(autouse=True)
+def _inference():
+    """These tests cover the fused forward; with autograd recording the module composes the
+    differentiable operators instead (tests/test_gpu_backward.py)."""
+    with torch.no_grad():
+        yield
+
+
 def _ops():
     from omni_moe.ops import hip
     return hip
