@@ -37,6 +37,16 @@ def expert_alg_bytes(T, H, k, s=2):
     return T * ((2 * k + 2) * H * s + k * (4 + s))
 
 
+def expert_bwd_alg_bytes(T, H, N, k, s=2):
+    """Backward of the expert op.  Token pass: x, dy and dx rows, k up rows, k down rows, k ids, gates and dgates,
+    k fp32 (ds, coef) pairs out.  Weight pass: per pair the x and dy rows, its two fp32 coefficients, pair id and token
+    id; the dU and dV tables out.  Plus the schedule."""
+    P = T * k
+    token_pass = T * (2 * k + 3) * H * s + P * (4 + 2 * s + 8)
+    weight_pass = P * (2 * H * s + 16) + 2 * N * H * s
+    return token_pass + weight_pass + P * 14 + 8 * (N + 1)
+
+
 def _events(torch, n):
     return [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
 
@@ -179,6 +189,11 @@ def main():
                                  expert_alg_bytes(T3, H, k), ms_seg3, "for comparison with expert_gather_kernel; same results"))
         out["roofline"] = max(kernels[:3], key=lambda d: d["kernel_ms"])
         out["roofline_expert"] = kernels[-3]
+        # training path (not part of the forward metric): backward of the expert op at the same shape
+        dy3 = x3 * 0.5
+        ms_b3 = time_call(torch, lambda: hip.hip_omni_expert_bwd_func(dy3, x3, up3, down3, g3, i3), reps)
+        kernels.append(hbm_entry("expert op backward (schedule + token pass + weight pass), c3", expert_bwd_alg_bytes(T3, H, N, k), ms_b3,
+                                 "x, dy (32 MiB each) and the tables are cache-resident, so algorithmic bytes exceed HBM traffic"))
         out["kernels"] = kernels
 
     if not a.no_cpu_baseline:

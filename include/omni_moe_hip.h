@@ -1,4 +1,4 @@
-/* C ABI of libomni_moe_hip.so: the OmniMoE forward path on AMD Instinct MI355X (gfx950).
+/* C ABI of libomni_moe_hip.so: the OmniMoE layer (forward path, plus the backward of its three operators) on AMD Instinct MI355X (gfx950).
  *
  * Plain pointers and sizes only.  Every pointer named "device" is a device address
  * of a densely packed row-major array.  Every call enqueues its kernels on `stream`

@@ -30,12 +30,11 @@ constexpr int kBwdWavesPerBlock = 4;
 __device__ __forceinline__ float sigmoid_f32(float x) { return 1.0f / (1.0f + __expf(-x)); }
 
 // ---- router ------------------------------------------------------------------------------------
-// One wave per token; lane l accumulates columns l, l+64, ... of both halves (r <= 1024).
-template <int DT>
+// One wave per token; lane l accumulates columns l, l+64, ... of both halves (r <= 64 * kCols).
+template <int DT, int kCols>
 __global__ __launch_bounds__(kBwdWavesPerBlock* kWave) void router_bwd_kernel(
     const void* __restrict__ dscores, const int32_t* __restrict__ ids, void* __restrict__ dlx, void* __restrict__ dly,
     int num_tokens, int r, int top_k) {
-  constexpr int kCols = 16;                         // 16 * 64 = 1024 columns per half
   const int lane = lane_id();
   const int t = __builtin_amdgcn_readfirstlane(blockIdx.x * kBwdWavesPerBlock + (threadIdx.x >> 6));
   if (t >= num_tokens) return;
@@ -47,12 +46,13 @@ __global__ __launch_bounds__(kBwdWavesPerBlock* kWave) void router_bwd_kernel(
     const int j = j0 + lane;
     const int my_id = j < top_k ? ids[base + j] : -1;
     const float my_ds = j < top_k ? Elem<DT>::load(dscores, base + j) : 0.f;
+    // lane j splits slot j's id once; an id outside the product gets coordinates no lane owns
+    const bool ok = (uint32_t)my_id < (uint32_t)r * (uint32_t)r;
+    const int my_ix = ok ? my_id / r : -1, my_iy = ok ? my_id - my_ix * r : -1;
     const int n = min(kWave, top_k - j0);
     for (int i = 0; i < n; ++i) {                   // slot order: the sum per column is deterministic
-      const int id = __shfl(my_id, i, kWave);
+      const int ix = __shfl(my_ix, i, kWave), iy = __shfl(my_iy, i, kWave);
       const float ds = __shfl(my_ds, i, kWave);
-      if ((uint32_t)id >= (uint32_t)r * (uint32_t)r) continue;   // uniform: an id outside the product is ignored
-      const int ix = id / r, iy = id - ix * r;
 #pragma unroll
       for (int c = 0; c < kCols; ++c) {
         ax[c] += (ix == c * kWave + lane) ? ds : 0.f;
@@ -293,9 +293,16 @@ extern "C" OMNI_API int32_t omni_router_bwd(const void* dscores, const int32_t* 
   dim3 grid((unsigned)((num_tokens + kBwdWavesPerBlock - 1) / kBwdWavesPerBlock)), block(kBwdWavesPerBlock * kWave);
   hipStream_t s = (hipStream_t)stream;
   const int T = (int)num_tokens, r = num_expert_sqrt, k = num_experts_per_token;
-  if (dtype == OMNI_BF16) hipLaunchKernelGGL(router_bwd_kernel<kBF16>, grid, block, 0, s, dscores, indices, dlogits_x, dlogits_y, T, r, k);
-  else if (dtype == OMNI_F16) hipLaunchKernelGGL(router_bwd_kernel<kF16>, grid, block, 0, s, dscores, indices, dlogits_x, dlogits_y, T, r, k);
-  else hipLaunchKernelGGL(router_bwd_kernel<kF32>, grid, block, 0, s, dscores, indices, dlogits_x, dlogits_y, T, r, k);
+#define OMNI_ROUTER_BWD_CASE(DT)                                                                                             \
+  do {                                                                                                                       \
+    if (r <= 64) hipLaunchKernelGGL((router_bwd_kernel<DT, 1>), grid, block, 0, s, dscores, indices, dlogits_x, dlogits_y, T, r, k);        \
+    else if (r <= 256) hipLaunchKernelGGL((router_bwd_kernel<DT, 4>), grid, block, 0, s, dscores, indices, dlogits_x, dlogits_y, T, r, k);  \
+    else hipLaunchKernelGGL((router_bwd_kernel<DT, 16>), grid, block, 0, s, dscores, indices, dlogits_x, dlogits_y, T, r, k);               \
+  } while (0)
+  if (dtype == OMNI_BF16) OMNI_ROUTER_BWD_CASE(kBF16);
+  else if (dtype == OMNI_F16) OMNI_ROUTER_BWD_CASE(kF16);
+  else OMNI_ROUTER_BWD_CASE(kF32);
+#undef OMNI_ROUTER_BWD_CASE
   return to_code(hipGetLastError());
 }
 
