@@ -164,17 +164,28 @@ __global__ __launch_bounds__(kBwdWavesPerBlock* kWave, 2) void expert_bwd_token_
 }
 
 // ---- experts, weight pass ----------------------------------------------------------------------
+// The sorted pair list is cut into chunks of `chunk` consecutive pairs, one wave each, whatever the
+// segment lengths: a popular expert's segment is spread over many waves and many rare experts
+// share one.  Inside its chunk a wave sums run after run (a run = the chunk's pairs of one
+// expert).  A run that is the expert's whole segment is rounded and stored straight away.  A run
+// of a segment that crosses the chunk's border is left as an fp32 partial row pair in
+// `partials[chunk][slot]`, slot 0 if the run starts the chunk, slot 1 otherwise (a chunk has at
+// most one of each); the fix-up kernel then adds an expert's partials in chunk order, so the
+// summation order is fixed and nothing is added atomically.
 template <int DT, int NCH, int G>
 __global__ __launch_bounds__(kBwdWavesPerBlock* kWave, 2) void expert_bwd_weight_kernel(
     const uint8_t* __restrict__ x, const uint8_t* __restrict__ dy, const float* __restrict__ ds, const float* __restrict__ coef,
-    const int32_t* __restrict__ offsets, const int32_t* __restrict__ sorted_pair_ids, const int32_t* __restrict__ sorted_token_ids,
-    uint8_t* __restrict__ dup, uint8_t* __restrict__ ddown, int64_t num_experts, int hidden) {
+    const int32_t* __restrict__ ids, const int32_t* __restrict__ offsets, const int32_t* __restrict__ sorted_pair_ids,
+    const int32_t* __restrict__ sorted_token_ids, uint8_t* __restrict__ dup, uint8_t* __restrict__ ddown,
+    float* __restrict__ partials, int64_t num_experts, int hidden, int chunk, int num_chunks) {
   constexpr int E = Row16<DT>::kElems;
   const int lane = lane_id();
-  const int64_t e = __builtin_amdgcn_readfirstlane((int)(blockIdx.x * kBwdWavesPerBlock + (threadIdx.x >> 6)));
-  if (e >= num_experts) return;
+  const int ci = __builtin_amdgcn_readfirstlane((int)(blockIdx.x * kBwdWavesPerBlock + (threadIdx.x >> 6)));
+  if (ci >= num_chunks) return;
+  const int valid = offsets[num_experts];             // pairs with an id inside the table
+  const int first = ci * chunk, last = min(first + chunk, valid);
+  if (first >= last) return;
   const int64_t row_bytes = int64_t(hidden) * (16 / E);
-  const int begin = offsets[e], end = offsets[e + 1];
 
   bool live[NCH];
   int64_t off[NCH];
@@ -186,17 +197,48 @@ __global__ __launch_bounds__(kBwdWavesPerBlock* kWave, 2) void expert_bwd_weight
 #pragma unroll
     for (int i = 0; i < E; ++i) au[c][i] = av[c][i] = 0.f;
   }
-  for (int p0 = begin; p0 < end; p0 += G) {          // segment order = pair order: a fixed summation order
+  // ends the run [run_first, run_last) of expert e and clears the accumulators
+  auto flush = [&](int e, int run_first, int run_last) {
+    const bool whole = offsets[e] == run_first && offsets[e + 1] == run_last;
+    if (whole) {
+#pragma unroll
+      for (int c = 0; c < NCH; ++c)
+        if (live[c]) {
+          *(u32x4_t*)(dup + e * row_bytes + off[c]) = pack16<DT>(au[c]);
+          *(u32x4_t*)(ddown + e * row_bytes + off[c]) = pack16<DT>(av[c]);
+        }
+    } else {
+      float* out = partials + (int64_t(ci) * 2 + (run_first == first ? 0 : 1)) * 2 * hidden;
+#pragma unroll
+      for (int c = 0; c < NCH; ++c)
+        if (live[c]) {
+          const int col = (c * kWave + lane) * E;
+#pragma unroll
+          for (int q = 0; q < E; q += 4) {
+            *(f32x4_t*)(out + col + q) = f32x4_t{au[c][q], au[c][q + 1], au[c][q + 2], au[c][q + 3]};
+            *(f32x4_t*)(out + hidden + col + q) = f32x4_t{av[c][q], av[c][q + 1], av[c][q + 2], av[c][q + 3]};
+          }
+        }
+    }
+#pragma unroll
+    for (int c = 0; c < NCH; ++c)
+#pragma unroll
+      for (int i = 0; i < E; ++i) au[c][i] = av[c][i] = 0.f;
+  };
+
+  int run_e = __builtin_amdgcn_readfirstlane(ids[sorted_pair_ids[first]]), run_first = first;
+  for (int p0 = first; p0 < last; p0 += G) {          // list order = (expert, pair) order: a fixed summation order
     int64_t tok[G];
+    int ee[G];
     float cs[G], cc[G];
 #pragma unroll
     for (int i = 0; i < G; ++i) {
-      const int p = min(p0 + i, end - 1);
+      const int p = min(p0 + i, last - 1);
       const int pid = sorted_pair_ids[p];
       tok[i] = sorted_token_ids[p];
-      const bool ok = p0 + i < end;
-      cs[i] = ok ? ds[pid] : 0.f;
-      cc[i] = ok ? coef[pid] : 0.f;
+      ee[i] = __builtin_amdgcn_readfirstlane(ids[pid]);
+      cs[i] = ds[pid];
+      cc[i] = coef[pid];
     }
     u32x4_t xr[G][NCH], dyr[G][NCH];
 #pragma unroll
@@ -207,18 +249,69 @@ __global__ __launch_bounds__(kBwdWavesPerBlock* kWave, 2) void expert_bwd_weight
         dyr[i][c] = live[c] ? *(const u32x4_t*)(dy + tok[i] * row_bytes + off[c]) : u32x4_t{0, 0, 0, 0};
       }
 #pragma unroll
-    for (int i = 0; i < G; ++i)
+    for (int i = 0; i < G; ++i) {
+      if (p0 + i >= last) break;
+      if (ee[i] != run_e) {
+        flush(run_e, run_first, p0 + i);
+        run_e = ee[i];
+        run_first = p0 + i;
+      }
 #pragma unroll
       for (int c = 0; c < NCH; ++c) {
         axpy16<DT>(cs[i], xr[i][c], au[c]);
         axpy16<DT>(cc[i], dyr[i][c], av[c]);
       }
+    }
+  }
+  flush(run_e, run_first, last);
+}
+
+// One wave per expert: zero rows for an expert nobody selected; for a segment that crosses a chunk
+// border the sum of its partial rows, first chunk to last.  A segment inside one chunk was
+// stored by the pass above.
+template <int DT, int NCH>
+__global__ __launch_bounds__(kBwdWavesPerBlock* kWave) void expert_bwd_weight_fixup_kernel(
+    const int32_t* __restrict__ offsets, const float* __restrict__ partials, uint8_t* __restrict__ dup,
+    uint8_t* __restrict__ ddown, int64_t num_experts, int hidden, int chunk) {
+  constexpr int E = Row16<DT>::kElems;
+  const int lane = lane_id();
+  const int64_t e = __builtin_amdgcn_readfirstlane((int)(blockIdx.x * kBwdWavesPerBlock + (threadIdx.x >> 6)));
+  if (e >= num_experts) return;
+  const int begin = offsets[e], end = offsets[e + 1];
+  const int c0 = begin / chunk, c1 = end > begin ? (end - 1) / chunk : c0;
+  if (end > begin && c0 == c1) return;
+  const int64_t row_bytes = int64_t(hidden) * (16 / E);
+  float au[NCH][E], av[NCH][E];
+#pragma unroll
+  for (int c = 0; c < NCH; ++c)
+#pragma unroll
+    for (int i = 0; i < E; ++i) au[c][i] = av[c][i] = 0.f;
+  if (end > begin) {
+    for (int ci = c0; ci <= c1; ++ci) {
+      const int slot = (ci == c0 && begin != c0 * chunk) ? 1 : 0;
+      const float* in = partials + (int64_t(ci) * 2 + slot) * 2 * hidden;
+#pragma unroll
+      for (int c = 0; c < NCH; ++c) {
+        const int col = (c * kWave + lane) * E;
+        if (col < hidden) {
+#pragma unroll
+          for (int q = 0; q < E; q += 4) {
+            const f32x4_t u = *(const f32x4_t*)(in + col + q), v = *(const f32x4_t*)(in + hidden + col + q);
+#pragma unroll
+            for (int z = 0; z < 4; ++z) {
+              au[c][q + z] += u[z];
+              av[c][q + z] += v[z];
+            }
+          }
+        }
+      }
+    }
   }
 #pragma unroll
   for (int c = 0; c < NCH; ++c)
-    if (live[c]) {
-      *(u32x4_t*)(dup + e * row_bytes + off[c]) = pack16<DT>(au[c]);
-      *(u32x4_t*)(ddown + e * row_bytes + off[c]) = pack16<DT>(av[c]);
+    if ((c * kWave + lane) * E < hidden) {
+      *(u32x4_t*)(dup + e * row_bytes + int64_t(c * kWave + lane) * 16) = pack16<DT>(au[c]);
+      *(u32x4_t*)(ddown + e * row_bytes + int64_t(c * kWave + lane) * 16) = pack16<DT>(av[c]);
     }
 }
 
@@ -259,11 +352,17 @@ __global__ __launch_bounds__(256) void swiglu_kernel(const uint8_t* __restrict__
 static inline size_t up256(size_t v) { return (v + 255) / 256 * 256; }
 static int to_code(hipError_t e) { return e == hipSuccess ? OMNI_OK : OMNI_ERR_HIP_BASE + (int)e; }
 
+// pairs per weight-pass chunk: about 2048 chunks (8 waves per CU), at least 16 pairs each
+static inline int weight_chunk(size_t pairs) {
+  const size_t c = (pairs + 2047) / 2048;
+  return (int)(c < 16 ? 16 : c);
+}
+
 template <int DT, int NCH, int G>
 static hipError_t launch_expert_bwd(const void* dy, const void* x, const void* up, const void* down, const void* gates,
                                     const int32_t* ids, void* dx, void* dup, void* ddown, void* dgates, float* ds, float* coef,
-                                    const int32_t* offsets, const int32_t* pair_ids, const int32_t* token_ids, int64_t T, int H,
-                                    int64_t N, int k, hipStream_t s) {
+                                    const int32_t* offsets, const int32_t* pair_ids, const int32_t* token_ids, float* partials,
+                                    int64_t T, int H, int64_t N, int k, hipStream_t s) {
   dim3 block(kBwdWavesPerBlock * kWave);
   if (T > 0) {
     dim3 grid((unsigned)((T + kBwdWavesPerBlock - 1) / kBwdWavesPerBlock));
@@ -272,9 +371,18 @@ static hipError_t launch_expert_bwd(const void* dy, const void* x, const void* u
                        (uint32_t)N);
     if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
   }
+  const size_t P = (size_t)T * (size_t)k;
+  const int chunk = weight_chunk(P);
+  const int num_chunks = (int)((P + chunk - 1) / chunk);
+  if (num_chunks > 0) {
+    dim3 grid((unsigned)((num_chunks + kBwdWavesPerBlock - 1) / kBwdWavesPerBlock));
+    hipLaunchKernelGGL((expert_bwd_weight_kernel<DT, NCH, G>), grid, block, 0, s, (const uint8_t*)x, (const uint8_t*)dy, ds, coef,
+                       ids, offsets, pair_ids, token_ids, (uint8_t*)dup, (uint8_t*)ddown, partials, N, H, chunk, num_chunks);
+    if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
+  }
   dim3 grid((unsigned)((N + kBwdWavesPerBlock - 1) / kBwdWavesPerBlock));
-  hipLaunchKernelGGL((expert_bwd_weight_kernel<DT, NCH, G>), grid, block, 0, s, (const uint8_t*)x, (const uint8_t*)dy, ds, coef,
-                     offsets, pair_ids, token_ids, (uint8_t*)dup, (uint8_t*)ddown, N, H);
+  hipLaunchKernelGGL((expert_bwd_weight_fixup_kernel<DT, NCH>), grid, block, 0, s, offsets, partials, (uint8_t*)dup,
+                     (uint8_t*)ddown, N, H, chunk);
   return hipGetLastError();
 }
 
@@ -306,15 +414,16 @@ extern "C" OMNI_API int32_t omni_router_bwd(const void* dscores, const int32_t* 
   return to_code(hipGetLastError());
 }
 
-// workspace: ds [P] f32 | coef [P] f32 | offsets [N+1] i32 | sorted pair ids [P] i32 | sorted token ids [P] i32 | schedule workspace
+// workspace: ds [P] f32 | coef [P] f32 | sorted pair ids [P] i32 | sorted token ids [P] i32 | offsets [N+1] i32 |
+//            partial rows [chunks][2][2][H] f32 | schedule workspace
 extern "C" OMNI_API size_t omni_expert_bwd_workspace_bytes(int64_t num_tokens, int32_t hidden_size, int64_t num_experts,
                                                            int32_t num_experts_per_token, int32_t dtype) {
   using namespace omni;
-  (void)hidden_size;
   (void)dtype;
-  if (num_tokens < 0 || num_experts <= 0 || num_experts_per_token < 0) return 0;
+  if (num_tokens < 0 || num_experts <= 0 || num_experts_per_token < 0 || hidden_size <= 0) return 0;
   const size_t P = (size_t)num_tokens * (size_t)num_experts_per_token;
-  return 4 * up256(P * 4) + up256(((size_t)num_experts + 1) * 4) +
+  const size_t chunks = (P + weight_chunk(P) - 1) / weight_chunk(P);
+  return 4 * up256(P * 4) + up256(((size_t)num_experts + 1) * 4) + up256(chunks * 4 * (size_t)hidden_size * 4) +
          omni_schedule_workspace_bytes(num_tokens, num_experts_per_token, num_experts);
 }
 
@@ -344,29 +453,30 @@ extern "C" OMNI_API int32_t omni_expert_bwd(const void* dy, const void* x, const
   int32_t* pair_ids = (int32_t*)w;     w += up256(P * 4);
   int32_t* token_ids = (int32_t*)w;    w += up256(P * 4);
   int32_t* offsets = (int32_t*)w;      w += up256(((size_t)num_experts + 1) * 4);
+  float* partials = (float*)w;
+  {
+    const size_t chunks = (P + weight_chunk(P) - 1) / weight_chunk(P);
+    w += up256(chunks * 4 * (size_t)hidden_size * 4);
+  }
   hipStream_t s = (hipStream_t)stream;
   if (int e = omni_schedule(indices, offsets, pair_ids, token_ids, num_tokens, num_experts_per_token, num_experts, w, stream)) return e;
   const int64_t T = num_tokens, N = num_experts;
   const int H = hidden_size, k = num_experts_per_token;
   hipError_t err;
-#define OMNI_BWD_CASE(DT)                                                                                                         \
-  do {                                                                                                                            \
-    if (nch <= 1) err = launch_expert_bwd<DT, 1, 8>(dy, x, up_weight, down_weight, routing_weights, indices, dx, dup_weight,     \
-                                                    ddown_weight, drouting_weights, ds, coef, offsets, pair_ids, token_ids, T,   \
-                                                    H, N, k, s);                                                                  \
-    else if (nch <= 2) err = launch_expert_bwd<DT, 2, 8>(dy, x, up_weight, down_weight, routing_weights, indices, dx,            \
-                                                         dup_weight, ddown_weight, drouting_weights, ds, coef, offsets,          \
-                                                         pair_ids, token_ids, T, H, N, k, s);                                    \
-    else if (nch <= 4) err = launch_expert_bwd<DT, 4, 4>(dy, x, up_weight, down_weight, routing_weights, indices, dx,            \
-                                                         dup_weight, ddown_weight, drouting_weights, ds, coef, offsets,          \
-                                                         pair_ids, token_ids, T, H, N, k, s);                                    \
-    else err = launch_expert_bwd<DT, 8, 2>(dy, x, up_weight, down_weight, routing_weights, indices, dx, dup_weight,              \
-                                           ddown_weight, drouting_weights, ds, coef, offsets, pair_ids, token_ids, T, H, N, k,   \
-                                           s);                                                                                    \
+#define OMNI_BWD_ARGS                                                                                                   \
+  dy, x, up_weight, down_weight, routing_weights, indices, dx, dup_weight, ddown_weight, drouting_weights, ds, coef, offsets, \
+      pair_ids, token_ids, partials, T, H, N, k, s
+#define OMNI_BWD_CASE(DT)                                                      \
+  do {                                                                         \
+    if (nch <= 1) err = launch_expert_bwd<DT, 1, 8>(OMNI_BWD_ARGS);            \
+    else if (nch <= 2) err = launch_expert_bwd<DT, 2, 8>(OMNI_BWD_ARGS);       \
+    else if (nch <= 4) err = launch_expert_bwd<DT, 4, 4>(OMNI_BWD_ARGS);       \
+    else err = launch_expert_bwd<DT, 8, 2>(OMNI_BWD_ARGS);                     \
   } while (0)
   if (dtype == OMNI_BF16) OMNI_BWD_CASE(kBF16);
   else if (dtype == OMNI_F16) OMNI_BWD_CASE(kF16);
   else OMNI_BWD_CASE(kF32);
+#undef OMNI_BWD_ARGS
 #undef OMNI_BWD_CASE
   return to_code(err);
 }

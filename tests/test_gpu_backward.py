@@ -84,7 +84,9 @@ def _expert_reference(x, up, down, gates, ids, dy):
     return y.detach(), x.grad, up.grad, down.grad, gates.grad
 
 
-EXPERT_BWD_CASES = [(256, 1024, 512, 16), (300, 256, 64, 8), (64, 2048, 128, 4), (33, 96, 16, 6), (128, 4096, 32, 2), (16, 64, 1024, 32)]
+# the last case has 65 600 pairs over 50 experts: every segment crosses dozens of the weight pass's chunks
+EXPERT_BWD_CASES = [(256, 1024, 512, 16), (300, 256, 64, 8), (64, 2048, 128, 4), (33, 96, 16, 6), (128, 4096, 32, 2), (16, 64, 1024, 32),
+                    (4100, 64, 50, 16)]
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
@@ -272,3 +274,26 @@ def test_layer_trains_bf16(device):
     with torch.no_grad():
         fused = layer(xd)
     torch.testing.assert_close(fused.float(), composed.float(), rtol=2e-2, atol=2e-2)
+
+
+def test_backward_edge_cases(device):
+    """No tokens, no slots: nothing to gather, weight gradients are all zero; argument errors are refused."""
+    hip = _ops()
+    H, N = 64, 32
+    up, down = torch.randn(N, H, device=device), torch.randn(N, H, device=device)
+    for T, k in ((0, 4), (5, 0)):
+        x, dy = torch.randn(T, H, device=device), torch.randn(T, H, device=device)
+        gates = torch.rand(T, k, device=device)
+        ids = torch.zeros(T, k, dtype=torch.int32, device=device)
+        dx, du, dv, dg = hip.hip_omni_expert_bwd_func(dy, x, up, down, gates, ids)
+        assert dx.shape == (T, H) and dg.shape == (T, k)
+        assert not du.any() and not dv.any() and not dx.any()
+        dlx, dly = hip.hip_omni_router_bwd_func(torch.randn(T, k, device=device), ids, 8)
+        assert dlx.shape == (T, 8) and not dlx.any() and not dly.any()
+    with pytest.raises(ValueError):
+        hip.hip_omni_expert_bwd_func(torch.randn(4, H + 8, device=device), torch.randn(4, H, device=device), up, down,
+                                     torch.rand(4, 2, device=device), torch.zeros(4, 2, dtype=torch.int32, device=device))
+    with pytest.raises(ValueError):
+        hip.hip_omni_router_bwd_func(torch.randn(4, 2, device=device), torch.zeros(4, 3, dtype=torch.int32, device=device), 8)
+    with pytest.raises(ValueError):                                   # r beyond what the kernel covers
+        hip.hip_omni_router_bwd_func(torch.randn(4, 2, device=device), torch.zeros(4, 2, dtype=torch.int32, device=device), 2048)
