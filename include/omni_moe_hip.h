@@ -5,8 +5,9 @@
  * (a hipStream_t passed as void*, NULL = the default stream) and returns without
  * waiting for the device.  The library allocates no memory: outputs and workspaces
  * come from the caller (the *_workspace_bytes calls give the sizes).  Inputs are
- * never written.  It keeps no mutable global state, so calls are re-entrant as long
- * as their outputs and workspaces are distinct.
+ * never written.  Its only global state is a per-kernel note of the devices whose
+ * shared-memory limit has been raised (atomic), so calls are re-entrant as long as
+ * their outputs and workspaces are distinct.
  *
  * Return value: OMNI_OK (0); a negative OMNI_ERR_* for a rejected argument (nothing
  * was enqueued); OMNI_ERR_HIP_BASE + hipError_t when the HIP runtime refused a launch.

@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 namespace omni {
 
 constexpr int kWave = 64;
@@ -79,6 +81,20 @@ __device__ __forceinline__ float silu_f32(float x) { return x / (1.0f + __expf(-
 // rounded to a 16-bit type straight away.
 __device__ __forceinline__ float silu_fast(float x) {
   return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(x * -1.4426950408889634f));
+}
+
+// ---- host side ---------------------------------------------------------------
+// Raises a kernel's dynamic-LDS limit, once per device (the attribute belongs to the device's
+// copy of the kernel).  `done` is that kernel's bit mask of devices already set up; concurrent
+// callers at worst set the attribute twice.
+inline hipError_t ensure_dynamic_lds(const void* kernel, int bytes, std::atomic<uint64_t>& done) {
+  int dev = 0;
+  if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
+  const uint64_t bit = 1ull << (dev & 63);
+  if (done.load(std::memory_order_acquire) & bit) return hipSuccess;
+  if (hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes); e != hipSuccess) return e;
+  done.fetch_or(bit, std::memory_order_release);
+  return hipSuccess;
 }
 
 }  // namespace omni

@@ -542,22 +542,14 @@ static hipError_t launch_gemm(GemmArgs g, hipStream_t s) {
     constexpr int kDmaLds = kDmaStages * (BM + BR) * kDmaBK * 2;
     static_assert(kDmaLds <= 160 * 1024, "LDS ring exceeds 160 KiB");
     auto kern = gemm_nt_dma_kernel<DT, TM, TN, EPI, kDmaBK, kDmaStages>;
-    static bool configured = false;                  // idempotent attribute, set once per instantiation
-    if (!configured) {
-      hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kDmaLds);
-      if (e != hipSuccess) return e;
-      configured = true;
-    }
+    static std::atomic<uint64_t> configured{0};      // one per kernel instantiation
+    if (hipError_t e = ensure_dynamic_lds((const void*)kern, kDmaLds, configured); e != hipSuccess) return e;
     hipLaunchKernelGGL(kern, dim3(blocks), dim3(kGemmThreads), kDmaLds, s, g);
     return hipGetLastError();
   }
   auto kern = gemm_nt_kernel<DT, TM, TN, EPI>;       // any K % 8 == 0: staged through registers
-  static bool configured = false;
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
-    if (e != hipSuccess) return e;
-    configured = true;
-  }
+  static std::atomic<uint64_t> configured{0};
+  if (hipError_t e = ensure_dynamic_lds((const void*)kern, kLds, configured); e != hipSuccess) return e;
   hipLaunchKernelGGL(kern, dim3(blocks), dim3(kGemmThreads), kLds, s, g);
   return hipGetLastError();
 }

@@ -279,13 +279,9 @@ extern "C" OMNI_API int32_t omni_schedule(const int32_t* indices, int32_t* offse
       a.top_k = num_experts_per_token;
       const int64_t entries = (int64_t)a.bins * a.blocks;
       const int scan_tiles = (int)((entries + kScanTile - 1) / kScanTile);
-      static bool configured = false;                      // tables of up to 4 x 4097 counters exceed the 64 KiB default
-      if (!configured) {
-        hipError_t e = hipFuncSetAttribute((const void*)sort_scatter_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                           kMaxBins * kSortWaves * 4);
-        if (e != hipSuccess) return OMNI_ERR_HIP_BASE + (int)e;
-        configured = true;
-      }
+      static std::atomic<uint64_t> configured{0};          // tables of up to 4 x 4097 counters exceed the 64 KiB default
+      if (hipError_t e = ensure_dynamic_lds((const void*)sort_scatter_kernel, kMaxBins * kSortWaves * 4, configured); e != hipSuccess)
+        return OMNI_ERR_HIP_BASE + (int)e;
       hipLaunchKernelGGL(sort_count_kernel, dim3(a.blocks), dim3(kSortThreads), (size_t)a.bins * 4, s, a);
       hipLaunchKernelGGL(scan_tiles_kernel, dim3(scan_tiles), dim3(kScanBlock), 0, s, hist, hist, tile_sums, entries);
       hipLaunchKernelGGL(scan_fixup_kernel, dim3(scan_tiles), dim3(kScanBlock), 0, s, hist, (int32_t*)nullptr, tile_sums, entries, scan_tiles);
