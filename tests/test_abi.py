@@ -100,3 +100,21 @@ def test_reference_import_paths():
     assert layer.num_expert_sqrt == 16 and layer.up_embed.weight.shape == (256, 64)
     with pytest.raises(ValueError):
         OmniMoE(OmniMoEConfig(64, 128, "gelu", 256, 8))
+
+
+def test_header_is_plain_c_and_a_c_program_links(tmp_path):
+    """The boundary is a C ABI: the header compiles as C99 (and C++), and a C program linked against the library
+    runs its host-side entry points without a GPU."""
+    inc = os.path.join(ROOT, "include")
+    for cmd in (["gcc", "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-fsyntax-only", "-x", "c", HEADER],
+                ["g++", "-std=c++17", "-Wall", "-Werror", "-fsyntax-only", "-x", "c++", HEADER]):
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        assert r.returncode == 0, r.stderr
+    lib = _lib().LIB_PATH
+    exe = str(tmp_path / "c_abi_client")
+    r = subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-I", inc, os.path.join(ROOT, "tests", "c_abi_client.c"), lib,
+                        "-Wl,-rpath," + os.path.dirname(lib), "-Wl,-rpath,/opt/rocm/lib", "-o", exe], capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
+    r = subprocess.run([exe], capture_output=True, text=True, timeout=60)
+    assert r.returncode == 0, (r.returncode, r.stdout, r.stderr)
+    assert "c abi ok" in r.stdout
