@@ -112,7 +112,7 @@ OMNI_API int32_t omni_expert_fwd(const void* x, const void* up_weight, const voi
  *   residual : NULL, or [T,H] added to the rounded down projection and rounded again
  *              (the layer's final  mlp + experts , omni_moe.py:102)
  *   workspace: omni_mlp_workspace_bytes() bytes (the [T,I] SwiGLU activations)
- * H and I must be multiples of 8 (of 4 for f32). */
+ * H and I must be multiples of 8 (of 4 for f32): rows are fetched 16 bytes at a time. */
 OMNI_API size_t omni_mlp_workspace_bytes(int64_t num_tokens, int32_t hidden_size, int32_t intermediate_size, int32_t dtype);
 OMNI_API int32_t omni_mlp_fwd(const void* x, const void* gate_weight, const void* up_weight, const void* down_weight,
                               const void* residual, void* y, int64_t num_tokens, int32_t hidden_size,
@@ -123,7 +123,8 @@ OMNI_API int32_t omni_mlp_fwd(const void* x, const void* gate_weight, const void
  * omni_linear_fwd:        y[T,out] = x[T,in] weight[out,in]^T [+ residual[T,out]]
  *                         (a bias-free nn.Linear / torch.matmul(., W.t()): interface.py:23-29,
  *                          omni_moe/modules/omni_moe.py:47-52,70-71)
- * in_features / hidden_size multiples of 8 (4 for f32), out_features / intermediate_size of 4. */
+ * in_features / hidden_size multiples of 8 (4 for f32); out_features / intermediate_size of any size
+ * (multiples of 8 take the widest stores). */
 OMNI_API int32_t omni_swiglu_linear_fwd(const void* x, const void* gate_weight, const void* up_weight, void* h,
                                         int64_t num_tokens, int32_t hidden_size, int32_t intermediate_size,
                                         int32_t dtype, void* stream);

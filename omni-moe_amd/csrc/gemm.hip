@@ -71,6 +71,7 @@ struct GemmArgs {           // all element offsets below are scaled by the eleme
   int tiles_m, tiles_n;
   int patch_m, patch_n;   // XCD patch shape (0 = plain order)
   int wide;               // 16-bit output: N % 8 == 0 and C 16-byte aligned, rows are written 16 bytes per lane
+  int single;             // N % 4 != 0: rows are not 8-byte aligned, results leave element by element
   float* part_mean;       // kEpiStats only: [ceil(M/32)][N] mean of each column over
   float* part_m2;         //   rows 32s..32s+31 of the ROUNDED result, and the sum of squared deviations
 };
@@ -192,11 +193,22 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, f32x16_t (&acc)
 #pragma unroll
       for (int q4 = 0; q4 < 4; ++q4) {
         const int n = nt + q4 * 8 + (lane >> 5) * 4;
-        if (n >= g.N) continue;                          // N is a multiple of 4
+        if (n >= g.N) continue;
         float v[4];
 #pragma unroll
         for (int q = 0; q < 4; ++q) v[q] = value(i, j, q4, q);
-        const int64_t o = ((int64_t)m * g.N + n) * ElemBytes<DT>::value;
+        if (g.single) {                                  // any N: one element at a time
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            if (n + q >= g.N) continue;
+            const int64_t at = (int64_t)m * g.N + n + q;
+            float out = v[q];
+            if constexpr (EPI == kEpiResidual) out = Elem<DT>::round(out) + Elem<DT>::load(g.res, at);
+            Elem<DT>::store(g.c, at, out);
+          }
+          continue;
+        }
+        const int64_t o = ((int64_t)m * g.N + n) * ElemBytes<DT>::value;   // N is a multiple of 4 here
         if constexpr (EPI == kEpiResidual) {
           // y = round(h Wd^T) + e, rounded again: the reference adds two stored tensors
           if constexpr (DT == kF32) {
@@ -530,6 +542,7 @@ static hipError_t launch_gemm(GemmArgs g, hipStream_t s) {
   // one XCD runs 32 blocks at a time: give it 4 x 8 patches when the tile grid allows
   g.patch_m = g.patch_n = 0;
   g.wide = (DT != kF32) && g.N % 8 == 0 && ((uintptr_t)g.c % 16 == 0);
+  g.single = g.N % 4 != 0;
   if (blocks % 256 == 0) {
     if (g.tiles_m % 4 == 0 && g.tiles_n % 8 == 0) { g.patch_m = 4; g.patch_n = 8; }
     else if (g.tiles_m % 8 == 0 && g.tiles_n % 4 == 0) { g.patch_m = 8; g.patch_n = 4; }
@@ -554,10 +567,10 @@ static hipError_t launch_gemm(GemmArgs g, hipStream_t s) {
   return hipGetLastError();
 }
 
-// Shape rules shared by the entry points: K a multiple of a 16-byte chunk, N of 4.
+// Shape rule shared by the entry points: K a multiple of a 16-byte chunk (rows are fetched 16 bytes at a time).
 static int check_gemm(int64_t M, int64_t N, int64_t K, int elem_bytes) {
   if (M < 0 || N <= 0 || K <= 0 || M > INT32_MAX / 2 || N > INT32_MAX / 2 || K > INT32_MAX / 2) return OMNI_ERR_SHAPE;
-  if (K % (16 / elem_bytes) != 0 || N % 4 != 0) return OMNI_ERR_SHAPE;
+  if (K % (16 / elem_bytes) != 0) return OMNI_ERR_SHAPE;
   return OMNI_OK;
 }
 
@@ -569,7 +582,7 @@ static int gemm_plain(const void* a, const void* b, const void* b_hi, const void
                       float* part_mean = nullptr, float* part_m2 = nullptr) {
   if (int e = check_gemm(M, N, K, ElemBytes<DT>::value)) return e;
   if (M == 0) return OMNI_OK;
-  GemmArgs g{(const uint8_t*)a, (const uint8_t*)b, (const uint8_t*)b_hi, (const uint8_t*)res, (uint8_t*)c, (int)M, (int)N, (int)K, 0, 0, 0, 0, 0, nullptr, nullptr};
+  GemmArgs g{(const uint8_t*)a, (const uint8_t*)b, (const uint8_t*)b_hi, (const uint8_t*)res, (uint8_t*)c, (int)M, (int)N, (int)K, 0, 0, 0, 0, 0, 0, nullptr, nullptr};
   g.part_mean = part_mean;
   g.part_m2 = part_m2;
   const int64_t big = ((M + 255) / 256) * ((N + 255) / 256), mid = ((M + 127) / 128) * ((N + 127) / 128);
@@ -594,7 +607,7 @@ template <int DT>
 static int gemm_swiglu(const void* x, const void* wg, const void* wu, void* h, int64_t M, int64_t I, int64_t K, hipStream_t s) {
   if (int e = check_gemm(M, I, K, ElemBytes<DT>::value)) return e;
   if (M == 0) return OMNI_OK;
-  GemmArgs g{(const uint8_t*)x, (const uint8_t*)wg, (const uint8_t*)wu, nullptr, (uint8_t*)h, (int)M, (int)I, (int)K, 0, 0, 0, 0, 0, nullptr, nullptr};
+  GemmArgs g{(const uint8_t*)x, (const uint8_t*)wg, (const uint8_t*)wu, nullptr, (uint8_t*)h, (int)M, (int)I, (int)K, 0, 0, 0, 0, 0, 0, nullptr, nullptr};
   const int64_t big = ((M + 255) / 256) * ((I + 127) / 128);
   hipError_t err;
   if (big >= 200) err = launch_gemm<DT, 4, 4, kEpiSwiglu>(g, s);

@@ -141,6 +141,9 @@ LAYER_CASES = [
     # (T, H, I, N, k, seed)
     (512, 256, 1024, 1024, 8, 0),      # BASELINE config 1 shape, in bf16
     (4096, 1024, 4096, 4096, 16, 3),   # BASELINE config 4 (README shape)
+    (300, 128, 256, 1000, 8, 1),       # N not a square: r = floor(sqrt(N)) = 31 (omni_moe.py:38), odd, ids < 961
+    (300, 128, 256, 1000, 40, 1),      # and k > r, so k' = r
+    (64, 64, 128, 50, 6, 2),           # r = 7
 ]
 
 
@@ -299,9 +302,10 @@ def test_add_inplace(device):
 
 
 # (M, N, K): the first five select the 128 x 128 output tiles (too few 256 x 256 tiles to fill the chip), ragged M
-# included; then a big-tile case, N % 8 == 4 (rows written 8 bytes per lane instead of 16) and a ragged last column tile
+# included; then a big-tile case, N % 8 == 4 (rows written 8 bytes per lane instead of 16), a ragged last column tile
 LINEAR_CASES = [(3300, 1024, 512), (3300, 1024, 640), (3300, 1024, 576), (4096, 1024, 4096), (2049, 1536, 1024),
-                (4096, 4096, 256), (300, 100, 264), (333, 1000, 256), (70, 4, 8)]
+                (4096, 4096, 256), (300, 100, 264), (333, 1000, 256), (70, 4, 8),
+                (300, 62, 128), (129, 1001, 64), (70, 6, 16), (5, 1, 8)]       # N % 4 != 0: element-wise stores
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
