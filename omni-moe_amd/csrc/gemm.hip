@@ -644,6 +644,11 @@ extern "C" OMNI_API int32_t omni_mlp_fwd(const void* x, const void* gate_weight,
   if (!workspace) return OMNI_ERR_WORKSPACE;
   hipStream_t s = (hipStream_t)stream;
   int e;
+  if (dtype != OMNI_BF16 && dtype != OMNI_F16 && dtype != OMNI_F32) return OMNI_ERR_DTYPE;
+  // both projections are checked before the first one is enqueued: hidden and intermediate size are each the K of one
+  const int es = dtype == OMNI_F32 ? 4 : 2;
+  if ((e = check_gemm(num_tokens, intermediate_size, hidden_size, es)) || (e = check_gemm(num_tokens, hidden_size, intermediate_size, es)))
+    return e;
   switch (dtype) {
     case OMNI_BF16:
       if ((e = gemm_swiglu<kBF16>(x, gate_weight, up_weight, workspace, num_tokens, intermediate_size, hidden_size, s))) return e;

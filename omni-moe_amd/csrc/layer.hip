@@ -35,6 +35,14 @@ extern "C" OMNI_API int32_t omni_moe_fwd(const void* x, const void* gate_weight,
   using namespace omni;
   if (num_tokens < 0 || hidden_size <= 0 || intermediate_size <= 0 || num_experts <= 0 || num_expert_sqrt <= 0) return OMNI_ERR_SHAPE;
   if (dtype != OMNI_BF16 && dtype != OMNI_F16 && dtype != OMNI_F32) return OMNI_ERR_DTYPE;
+  // every stage's shape rule, before the first kernel is enqueued
+  {
+    const int64_t esz = (int64_t)elem_bytes(dtype), r = num_expert_sqrt, k = num_experts_per_token;
+    if ((hidden_size * esz) % 16 != 0 || (intermediate_size * esz) % 16 != 0) return OMNI_ERR_SHAPE;   // rows are fetched 16 bytes at a time
+    if (k < 0 || k > r * r || k > 128 || k % 2 != 0) return OMNI_ERR_TOPK;
+    if (r > 1024 || hidden_size * esz > 8192) return OMNI_ERR_UNSUPPORTED;
+    if (r * r > num_experts) return OMNI_ERR_SHAPE;                                                   // ids reach r*r - 1
+  }
   if (num_tokens == 0) return OMNI_OK;
   if (!x || !y || !up_embed || !down_embed) return OMNI_ERR_NULL;
   if (!workspace) return OMNI_ERR_WORKSPACE;

@@ -71,6 +71,15 @@ def test_argument_errors_need_no_gpu():
     assert lib.omni_schedule(p, p, p, p, 4, 2, 0, p, None) == -2
     assert lib.omni_schedule(p, p, p, p, 4, 2, 16, None, None) == -6
     assert lib.omni_mlp_fwd(p, p, p, p, None, p, 4, 64, 62, 0, p, None) == -2   # intermediate size not a multiple of 8
+    # the whole layer: every stage's rule is checked before anything is enqueued
+    moe = lambda H, I, N, r, k, dt=0: lib.omni_moe_fwd(*([p] * 15), 4, H, I, N, r, k, dt, 2, 0, 0.1, 1e-5, p, None, None, None, None)
+    assert moe(64, 62, 16, 4, 2) == -2           # intermediate size
+    assert moe(60, 64, 16, 4, 2) == -2           # hidden size
+    assert moe(64, 64, 16, 4, 3) == -4           # odd k
+    assert moe(64, 64, 16, 4, 18) == -4          # k > r*r
+    assert moe(64, 64, 15, 4, 2) == -2           # r*r experts do not fit the tables
+    assert moe(8192, 64, 16, 4, 2) == -5         # rows beyond 8 KiB
+    assert moe(64, 64, 16, 4, 2, dt=5) == -3
     assert lib.omni_mlp_fwd(p, p, p, p, None, p, 4, 64, 64, 0, None, None) == -6 # no workspace
     assert lib.omni_schedule_workspace_bytes(4, 2, 100) >= 400
 
