@@ -3,7 +3,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
 Prints ONE JSON line.  A step = one forward of the OmniMoE layer over one batch of synthetic,
-HBM-resident input: BASELINE config 4, the README shape (1 x 4096 tokens, hidden 1024,
+HBM-resident input: benchmark config 4, the README shape (1 x 4096 tokens, hidden 1024,
 intermediate 4096, 4096 experts = 64 x 64 keys, top-16, bf16, train-mode BatchNorm).
 All timing uses HIP events recorded on the stream the kernels run on (torch's current stream;
 the library enqueues there).
@@ -12,7 +12,7 @@ the library enqueues there).
   roofline   the kernel that takes the largest share of a step (gate/up MFMA GEMM), timed per
              launch with events around its C-ABI call
   kernels    the same per-launch figures for every stage of the step, plus the fused expert
-             kernel on BASELINE config 3 (16384 tokens), the shape its bandwidth target is quoted on
+             kernel on benchmark config 3 (16384 tokens), the shape its bandwidth target is quoted on
 """
 import argparse
 import json
@@ -102,7 +102,7 @@ def main():
     torch.cuda.set_device(dev)
     torch.set_grad_enabled(False)          # forward path: the module then issues its single fused library call
 
-    # ---------------- BASELINE config 4: README-shape full layer
+    # ---------------- benchmark config 4: README-shape full layer
     T, H, I, N, k, seed = 4096, 1024, 4096, 4096, 16, 3
     x, w = oracle.make_layer_inputs(seed, T, H, I, N)
     layer = OmniMoE(OmniMoEConfig(H, I, "silu", N, k))
@@ -131,7 +131,7 @@ def main():
         "value": T / (ms_per_step * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": "BASELINE config 4: full OmniMoE layer forward, 1x4096 tokens, hidden 1024, intermediate 4096, "
+        "config": {"workload": "BASELINE.json configs[3] (benchmark config 4, the README shape): full OmniMoE layer forward, 1x4096 tokens, hidden 1024, intermediate 4096, "
                                "4096 experts (64x64), top-16, silu, train-mode BatchNorm, seed 3"},
         "wall_s_timed_region": wall,
     }
@@ -175,7 +175,7 @@ def main():
             {"kernel": "router stage (projection GEMM with BN statistics epilogue + BN finalize + select), c4", "kernel_ms": ms_router,
              "algorithmic_flops": 4 * T * H * r},
         ]
-        # expert kernel at the shape its bandwidth target is quoted on (BASELINE config 3)
+        # expert kernel at the shape its bandwidth target is quoted on (benchmark config 3)
         T3 = 16384
         x3, up3, down3, g3, i3 = (t.to(dev) for t in oracle.make_expert_inputs(2, T3, H, N, k))
         ms_e3 = time_call(torch, lambda: hip.hip_omni_expert_func(x3, up3, down3, g3, i3), reps)

@@ -139,8 +139,8 @@ def test_router_fwd_select_is_exact_given_same_logprobs(device):
 
 LAYER_CASES = [
     # (T, H, I, N, k, seed)
-    (512, 256, 1024, 1024, 8, 0),      # BASELINE config 1 shape, in bf16
-    (4096, 1024, 4096, 4096, 16, 3),   # BASELINE config 4 (README shape)
+    (512, 256, 1024, 1024, 8, 0),      # benchmark config 1 shape, in bf16
+    (4096, 1024, 4096, 4096, 16, 3),   # benchmark config 4 (README shape)
     (300, 128, 256, 1000, 8, 1),       # N not a square: r = floor(sqrt(N)) = 31 (omni_moe.py:38), odd, ids < 961
     (300, 128, 256, 1000, 40, 1),      # and k > r, so k' = r
     (64, 64, 128, 50, 6, 2),           # r = 7
@@ -183,7 +183,7 @@ def test_layer_matches_oracle(case, training, device):
 
 @pytest.mark.parametrize("training", [True, False], ids=["train", "eval"])
 def test_layer_config1_fp32(training, device):
-    """BASELINE config 1, the reference's CPU-runnable case, at full size in fp32:
+    """benchmark config 1, the reference's CPU-runnable case, at full size in fp32:
     1 x 512 tokens, hidden 256, intermediate 1024, 1024 experts (32 x 32), top-8, seed 0."""
     from omni_moe.modules.omni_moe import OmniMoE, OmniMoEConfig
     T, H, I, N, k = 512, 256, 1024, 1024, 8
@@ -216,7 +216,7 @@ def test_layer_config1_fp32(training, device):
 
 
 def test_layer_config5_large_skewed(device):
-    """BASELINE config 5: 8 x 4096 tokens, hidden 2048, intermediate 8192, 262144 experts
+    """benchmark config 5: 8 x 4096 tokens, hidden 2048, intermediate 8192, 262144 experts
     (512 x 512 keys), top-32, bf16, router key popularity ~ Zipf(1.1), seed 4.
 
     The reference's router has no bias (omni_moe.py:47-52), so the per-key bias b_i = -1.1*ln(1+i)

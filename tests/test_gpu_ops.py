@@ -27,9 +27,9 @@ ROUTER_CASES = [
     (1024, 128, 32, torch.bfloat16, "randn"),
     (1024, 256, 16, torch.bfloat16, "randn"),
     (1024, 256, 32, torch.bfloat16, "randn"),
-    (4096, 64, 16, torch.bfloat16, "logprob"),     # BASELINE config 2 shape
-    (2048, 512, 32, torch.bfloat16, "logprob"),    # BASELINE config 5 shape (token subset)
-    (512, 32, 8, torch.float32, "logprob"),        # BASELINE config 1 shape
+    (4096, 64, 16, torch.bfloat16, "logprob"),     # benchmark config 2 shape
+    (2048, 512, 32, torch.bfloat16, "logprob"),    # benchmark config 5 shape (token subset)
+    (512, 32, 8, torch.float32, "logprob"),        # benchmark config 1 shape
     (333, 64, 16, torch.float16, "randn"),
     (257, 100, 10, torch.bfloat16, "randn"),       # r not a multiple of 64
     (64, 4, 16, torch.bfloat16, "randn"),          # k = r*r: every expert selected, k' = r
@@ -124,9 +124,9 @@ EXPERT_CASES = [
     # (T, H, N, k, dtype, kind)
     (1024, 1024, 1024, 32, torch.bfloat16, "ref"),      # reference benchmark grid (tests/test_expert.py:181-187)
     (1024, 1024, 4096, 32, torch.bfloat16, "ref"),
-    (2048, 1024, 4096, 16, torch.bfloat16, "baseline"), # BASELINE config 3 shape (token subset)
-    (512, 256, 1024, 8, torch.float32, "baseline"),     # BASELINE config 1 shape
-    (256, 2048, 8192, 32, torch.bfloat16, "baseline"),  # BASELINE config 5 row length
+    (2048, 1024, 4096, 16, torch.bfloat16, "baseline"), # benchmark config 3 shape (token subset)
+    (512, 256, 1024, 8, torch.float32, "baseline"),     # benchmark config 1 shape
+    (256, 2048, 8192, 32, torch.bfloat16, "baseline"),  # benchmark config 5 row length
     (130, 1024, 512, 6, torch.float16, "ref"),
     (77, 520, 300, 10, torch.bfloat16, "ref"),          # H not a multiple of 512
     (64, 4096, 256, 4, torch.bfloat16, "ref"),

@@ -242,7 +242,7 @@ class _TorchLayer(nn.Module):
 
 @pytest.mark.parametrize("training", [True, False])
 def test_moe_forward_matches_torch_layer_fp32(training):
-    """BASELINE config 1 (the reference's CPU-runnable case) at reduced size, fp32."""
+    """benchmark config 1 (the reference's CPU-runnable case) at reduced size, fp32."""
     T, H, I, N, k = 128, 64, 256, 256, 8
     x, w = oracle.make_layer_inputs(0, T, H, I, N, dtype=torch.float32)
     layer = _TorchLayer(H, I, N, k)
@@ -265,7 +265,7 @@ def test_moe_forward_matches_torch_layer_fp32(training):
 
 
 def test_moe_forward_config1_full_size_runs():
-    """BASELINE config 1 at full size (T=512, H=256, I=1024, N=1024, k=8, fp32, seed 0)."""
+    """benchmark config 1 at full size (T=512, H=256, I=1024, N=1024, k=8, fp32, seed 0)."""
     x, w = oracle.make_layer_inputs(0, 512, 256, 1024, 1024, dtype=torch.float32)
     bx, by = oracle.BNState.fresh(32), oracle.BNState.fresh(32)
     y, gates, ids = oracle.moe_forward(x, w, bx, by, 8, training=True)
