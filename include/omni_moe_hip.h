@@ -148,6 +148,22 @@ OMNI_API int32_t omni_router_bwd(const void* dscores, const int32_t* indices, vo
                                  int64_t num_tokens, int32_t num_expert_sqrt, int32_t num_experts_per_token,
                                  int32_t dtype, void* stream);
 
+/* The rest of the router stage in reverse: from d(gates) back to d(z), z = x [Wx;Wy]^T being the
+ * raw projections that omni_router_fwd leaves in its workspace.  Covers what autograd does in the
+ * reference for torch.exp, the router op, F.log_softmax and nn.BatchNorm1d (omni_moe.py:70-86):
+ *   d(score) = d(gate) gate;  d(l) by omni_router_bwd's scatter;  d(n) = d(l) - exp(l) sum(d(l));
+ *   eval: d(z) = rstd d(n);   train: d(z) = rstd (d(n) - mean_T d(n) - nhat mean_T(d(n) nhat)).
+ *   dgates, gates [T,k] dtype `dtype`; indices [T,k] int32; z [T,2r] dtype `dtype` and stats [4r] f32
+ *   (mean_x | rstd_x | mean_y | rstd_y) as left by omni_router_fwd at workspace offset 0 and
+ *   omni_router_workspace_stats_offset(); dz [T,2r] dtype `dtype`, fully overwritten.
+ * The two GEMMs around it (dW = dz^T x, dx = dz [Wx;Wy]) are the caller's. */
+OMNI_API size_t omni_router_workspace_stats_offset(int64_t num_tokens, int32_t num_expert_sqrt, int32_t dtype);
+OMNI_API size_t omni_router_norm_bwd_workspace_bytes(int64_t num_tokens, int32_t num_expert_sqrt);
+OMNI_API int32_t omni_router_norm_bwd(const void* dgates, const void* gates, const int32_t* indices, const void* z,
+                                      const float* stats, void* dz, int64_t num_tokens, int32_t num_expert_sqrt,
+                                      int32_t num_experts_per_token, int32_t dtype, int32_t training, void* workspace,
+                                      void* stream);
+
 /* Fused atomic-expert backward.  For pair (t, e = indices[t,j]) with s = <x_t, U_e>, a = <dy_t, V_e>,
  * g = routing_weights[t,j]:  drouting_weights[t,j] = a silu(s);  dx_t += a g silu'(s) U_e;
  * dup_weight[e] += a g silu'(s) x_t;  ddown_weight[e] += silu(s) g dy_t.

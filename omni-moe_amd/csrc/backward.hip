@@ -70,6 +70,151 @@ __global__ __launch_bounds__(kBwdWavesPerBlock* kWave) void router_bwd_kernel(
   }
 }
 
+// ---- router stage: exp, Cartesian select, log-softmax and BatchNorm in reverse -------------------
+// The layer's router forward (omni_moe.py:70-86) is  z = x W^T -> n = BN(z) -> l = log_softmax(n)
+// -> scores = lx[ix] + ly[iy] -> gates = exp(scores).  Given d(gates), this pass returns d(z); the
+// two GEMMs around it (dW = dz^T x, dx = dz W) are the caller's.  One wave owns a token and walks
+// both halves with lane = column (R columns per lane and half):
+//   d(score_j) = d(gate_j) gate_j;  d(l) = scatter of d(score) by (ix, iy), in slot order;
+//   d(n) = d(l) - exp(l) sum(d(l));                      (log-softmax)
+//   eval:  d(z) = rstd d(n);   train:  d(z) = rstd (d(n) - mean_T d(n) - nhat mean_T(d(n) nhat)).
+// Training needs the two column means over all tokens: the first kernel leaves d(n) in the dz
+// buffer and per-block column sums, a one-wave-per-column kernel adds those, a third kernel
+// finishes d(z).  Values are rounded to the storage dtype where the reference's torch ops round
+// (d(score), d(l), d(n), d(z)); n and l are recomputed from z and the saved statistics.
+constexpr int kNormTokensPerWave = 8;
+
+template <int DT, int R>
+__global__ __launch_bounds__(kBwdWavesPerBlock* kWave) void router_norm_bwd_kernel(
+    const void* __restrict__ dgates, const void* __restrict__ gates, const int32_t* __restrict__ ids,
+    const void* __restrict__ z, const float* __restrict__ stats, void* __restrict__ dz, float* __restrict__ partials,
+    int num_tokens, int r, int top_k, int training) {
+  __shared__ float red[kBwdWavesPerBlock][4][R * kWave];       // per wave: S1x, S2x, S1y, S2y by column
+  const int lane = lane_id(), wave = threadIdx.x >> 6;
+  const int first = (blockIdx.x * kBwdWavesPerBlock + wave) * kNormTokensPerWave;
+  float s1[2][R], s2[2][R];
+#pragma unroll
+  for (int h = 0; h < 2; ++h)
+#pragma unroll
+    for (int a = 0; a < R; ++a) s1[h][a] = s2[h][a] = 0.f;
+  float mean[2][R], rstd[2][R];
+#pragma unroll
+  for (int h = 0; h < 2; ++h)
+#pragma unroll
+    for (int a = 0; a < R; ++a) {
+      const int key = a * kWave + lane;
+      mean[h][a] = key < r ? stats[(2 * h) * r + key] : 0.f;
+      rstd[h][a] = key < r ? stats[(2 * h + 1) * r + key] : 0.f;
+    }
+  for (int t = first; t < min(first + kNormTokensPerWave, num_tokens); ++t) {
+    // d(l): scatter of the slot gradients, fp32 sums in slot order, one rounding
+    float dl[2][R];
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int a = 0; a < R; ++a) dl[h][a] = 0.f;
+    const int64_t base = int64_t(t) * top_k;
+    for (int j0 = 0; j0 < top_k; j0 += kWave) {
+      const int j = j0 + lane;
+      const int my_id = j < top_k ? ids[base + j] : -1;
+      const float my_ds = j < top_k ? Elem<DT>::round(Elem<DT>::load(dgates, base + j) * Elem<DT>::load(gates, base + j)) : 0.f;
+      const bool ok = (uint32_t)my_id < (uint32_t)r * (uint32_t)r;
+      const int my_ix = ok ? my_id / r : -1, my_iy = ok ? my_id - my_ix * r : -1;
+      const int n = min(kWave, top_k - j0);
+      for (int i = 0; i < n; ++i) {
+        const int ix = __shfl(my_ix, i, kWave), iy = __shfl(my_iy, i, kWave);
+        const float ds = __shfl(my_ds, i, kWave);
+#pragma unroll
+        for (int a = 0; a < R; ++a) {
+          dl[0][a] += (ix == a * kWave + lane) ? ds : 0.f;
+          dl[1][a] += (iy == a * kWave + lane) ? ds : 0.f;
+        }
+      }
+    }
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      // recompute nhat (fp32), n = round(nhat), l = round(log_softmax(n))
+      float nhat[R], l[R];
+      float m = -INFINITY;
+#pragma unroll
+      for (int a = 0; a < R; ++a) {
+        const int key = a * kWave + lane;
+        const float zv = key < r ? Elem<DT>::load(z, int64_t(t) * 2 * r + h * r + key) : 0.f;
+        nhat[a] = (zv - mean[h][a]) * rstd[h][a];
+        l[a] = key < r ? Elem<DT>::round(nhat[a]) : -INFINITY;
+        m = fmaxf(m, l[a]);
+      }
+      m = wave_max(m);
+      float e = 0.f;
+#pragma unroll
+      for (int a = 0; a < R; ++a) e += (a * kWave + lane < r) ? expf(l[a] - m) : 0.f;
+      const float lse = logf(wave_sum(e));
+      float sum_dl = 0.f;
+#pragma unroll
+      for (int a = 0; a < R; ++a) {
+        dl[h][a] = Elem<DT>::round(dl[h][a]);
+        sum_dl += dl[h][a];
+      }
+      sum_dl = wave_sum(sum_dl);
+#pragma unroll
+      for (int a = 0; a < R; ++a) {
+        const int key = a * kWave + lane;
+        if (key >= r) continue;
+        const float p = expf(Elem<DT>::round(l[a] - m - lse));
+        const float dn = Elem<DT>::round(dl[h][a] - p * sum_dl);
+        s1[h][a] += dn;
+        s2[h][a] += dn * nhat[a];
+        Elem<DT>::store(dz, int64_t(t) * 2 * r + h * r + key, training ? dn : dn * rstd[h][a]);
+      }
+    }
+  }
+  if (!training) return;
+  // column sums of the block: waves in order through LDS, then one row of partials per block
+#pragma unroll
+  for (int h = 0; h < 2; ++h)
+#pragma unroll
+    for (int a = 0; a < R; ++a) {
+      red[wave][2 * h][a * kWave + lane] = s1[h][a];
+      red[wave][2 * h + 1][a * kWave + lane] = s2[h][a];
+    }
+  __syncthreads();
+  for (int i = threadIdx.x; i < 4 * R * kWave; i += kBwdWavesPerBlock * kWave) {
+    const int q = i / (R * kWave), col = i % (R * kWave);
+    if (col >= r) continue;
+    float acc = 0.f;
+#pragma unroll
+    for (int w = 0; w < kBwdWavesPerBlock; ++w) acc += red[w][q][col];
+    partials[(int64_t(blockIdx.x) * 4 + q) * r + col] = acc;     // [block][S1x, S2x, S1y, S2y][r]
+  }
+}
+
+// means[q][col] = sum over blocks of partials / T; one wave per (q, col)
+__global__ __launch_bounds__(kBwdWavesPerBlock* kWave) void router_norm_bwd_sums_kernel(
+    const float* __restrict__ partials, float* __restrict__ means, int blocks, int r, int num_tokens) {
+  const int lane = lane_id();
+  const int idx = blockIdx.x * kBwdWavesPerBlock + (threadIdx.x >> 6);      // q * r + col
+  if (idx >= 4 * r) return;
+  double acc = 0.;
+  for (int b = lane; b < blocks; b += kWave) acc += (double)partials[int64_t(b) * 4 * r + idx];
+#pragma unroll
+  for (int m = kWave / 2; m >= 1; m >>= 1) acc += __shfl_xor(acc, m, kWave);
+  if (lane == 0) means[idx] = (float)(acc / (double)num_tokens);
+}
+
+// dz = rstd (dn - mean(dn) - nhat mean(dn nhat)), element-wise over [T, 2r]; dn is read from dz
+template <int DT>
+__global__ __launch_bounds__(256) void router_norm_bwd_finish_kernel(const void* __restrict__ z, const float* __restrict__ stats,
+                                                                    const float* __restrict__ means, void* __restrict__ dz,
+                                                                    int64_t num_values, int r) {
+  for (int64_t i = blockIdx.x * 256ll + threadIdx.x; i < num_values; i += gridDim.x * 256ll) {
+    const int c = (int)(i % (2 * r)), h = c >= r, key = c - h * r;
+    const float mu = stats[(2 * h) * r + key], rs = stats[(2 * h + 1) * r + key];
+    const float nhat = (Elem<DT>::load(z, i) - mu) * rs;
+    const float dn = Elem<DT>::load(dz, i);
+    Elem<DT>::store(dz, i, rs * (dn - means[(2 * h) * r + key] - nhat * means[(2 * h + 1) * r + key]));
+  }
+}
+
 // ---- experts, token pass -----------------------------------------------------------------------
 template <int DT, int NCH, int G>
 __global__ __launch_bounds__(kBwdWavesPerBlock* kWave, 2) void expert_bwd_token_kernel(
@@ -411,6 +556,60 @@ extern "C" OMNI_API int32_t omni_router_bwd(const void* dscores, const int32_t* 
   else if (dtype == OMNI_F16) OMNI_ROUTER_BWD_CASE(kF16);
   else OMNI_ROUTER_BWD_CASE(kF32);
 #undef OMNI_ROUTER_BWD_CASE
+  return to_code(hipGetLastError());
+}
+
+// workspace of omni_router_norm_bwd: per-block column sums [blocks][4][r] f32 | means [4][r] f32
+static inline int norm_bwd_blocks(int64_t num_tokens) {
+  const int64_t per_block = (int64_t)omni::kBwdWavesPerBlock * omni::kNormTokensPerWave;
+  return (int)((num_tokens + per_block - 1) / per_block);
+}
+
+extern "C" OMNI_API size_t omni_router_norm_bwd_workspace_bytes(int64_t num_tokens, int32_t num_expert_sqrt) {
+  using namespace omni;
+  if (num_tokens < 0 || num_expert_sqrt <= 0) return 0;
+  return up256((size_t)norm_bwd_blocks(num_tokens) * 4 * num_expert_sqrt * 4) + up256((size_t)4 * num_expert_sqrt * 4);
+}
+
+extern "C" OMNI_API int32_t omni_router_norm_bwd(const void* dgates, const void* gates, const int32_t* indices, const void* z,
+                                                 const float* stats, void* dz, int64_t num_tokens, int32_t num_expert_sqrt,
+                                                 int32_t num_experts_per_token, int32_t dtype, int32_t training, void* workspace,
+                                                 void* stream) {
+  using namespace omni;
+  const int r = num_expert_sqrt, k = num_experts_per_token;
+  if (num_tokens < 0 || num_tokens > INT32_MAX / 4096 || r <= 0 || k < 0) return OMNI_ERR_SHAPE;
+  if (r > 1024) return OMNI_ERR_UNSUPPORTED;
+  if (k > 128) return OMNI_ERR_TOPK;
+  if (dtype != OMNI_BF16 && dtype != OMNI_F16 && dtype != OMNI_F32) return OMNI_ERR_DTYPE;
+  if (num_tokens == 0) return OMNI_OK;
+  if (!z || !stats || !dz || (k > 0 && (!dgates || !gates || !indices))) return OMNI_ERR_NULL;
+  if (training && !workspace) return OMNI_ERR_WORKSPACE;
+  hipStream_t s = (hipStream_t)stream;
+  const int T = (int)num_tokens, blocks = norm_bwd_blocks(num_tokens);
+  float* partials = (float*)workspace;
+  float* means = training ? (float*)((char*)workspace + up256((size_t)blocks * 4 * r * 4)) : nullptr;
+  dim3 block(kBwdWavesPerBlock * kWave);
+#define OMNI_NORM_CASE(DT)                                                                                                    \
+  do {                                                                                                                        \
+    if (r <= 64) hipLaunchKernelGGL((router_norm_bwd_kernel<DT, 1>), dim3(blocks), block, 0, s, dgates, gates, indices, z,     \
+                                    stats, dz, partials, T, r, k, training);                                                   \
+    else if (r <= 256) hipLaunchKernelGGL((router_norm_bwd_kernel<DT, 4>), dim3(blocks), block, 0, s, dgates, gates, indices,  \
+                                          z, stats, dz, partials, T, r, k, training);                                          \
+    else hipLaunchKernelGGL((router_norm_bwd_kernel<DT, 16>), dim3(blocks), block, 0, s, dgates, gates, indices, z, stats, dz, \
+                            partials, T, r, k, training);                                                                      \
+    if (training) {                                                                                                           \
+      hipLaunchKernelGGL(router_norm_bwd_sums_kernel, dim3((4 * r + kBwdWavesPerBlock - 1) / kBwdWavesPerBlock), block, 0, s,  \
+                         partials, means, blocks, r, T);                                                                       \
+      const int64_t values = (int64_t)T * 2 * r;                                                                              \
+      const int64_t want = (values + 255) / 256;                                                                              \
+      hipLaunchKernelGGL(router_norm_bwd_finish_kernel<DT>, dim3((unsigned)(want < 4096 ? want : 4096)), dim3(256), 0, s, z,   \
+                         stats, means, dz, values, r);                                                                         \
+    }                                                                                                                         \
+  } while (0)
+  if (dtype == OMNI_BF16) OMNI_NORM_CASE(kBF16);
+  else if (dtype == OMNI_F16) OMNI_NORM_CASE(kF16);
+  else OMNI_NORM_CASE(kF32);
+#undef OMNI_NORM_CASE
   return to_code(hipGetLastError());
 }
 

@@ -622,6 +622,15 @@ extern "C" OMNI_API size_t omni_router_workspace_bytes(int64_t num_tokens, int32
   return align256((size_t)num_tokens * 2 * r * es) + align256(4 * r * 4) + 2 * align256(strips * 2 * r * 4);
 }
 
+// After omni_router_fwd the workspace still holds what a backward pass needs: z at offset 0 and,
+// at this offset, the fp32 statistics [mean_x | rstd_x | mean_y | rstd_y], r values each.
+extern "C" OMNI_API size_t omni_router_workspace_stats_offset(int64_t num_tokens, int32_t num_expert_sqrt, int32_t dtype) {
+  using namespace omni;
+  if (num_tokens < 0 || num_expert_sqrt <= 0) return 0;
+  const size_t es = dtype == OMNI_F32 ? 4 : 2;
+  return align256((size_t)num_tokens * 2 * (size_t)num_expert_sqrt * es);
+}
+
 extern "C" OMNI_API int32_t omni_router_fwd(const void* x, const void* weight_x, const void* weight_y,
                                             void* running_mean_x, void* running_var_x, int64_t* num_batches_tracked_x,
                                             void* running_mean_y, void* running_var_y, int64_t* num_batches_tracked_y,

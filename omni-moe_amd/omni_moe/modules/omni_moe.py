@@ -8,8 +8,8 @@ caller's stream, joined by the final add (``overlap_branches = False``: everythi
 caller's stream, the add fused into the down projection).
 
 When autograd is recording and the input or a parameter requires grad, ``forward`` instead
-composes the differentiable operators exactly as the reference's forward does
-(omni_moe.py:64-104: Linear -> BatchNorm1d -> log_softmax -> router op -> exp -> expert op,
+composes differentiable operators in the reference's order (omni_moe.py:64-104: the router
+stage -- Linear, BatchNorm1d, log_softmax, router op, exp -- as one node, the expert op, the
 MLP op, add), so the layer trains; call it under ``torch.no_grad()`` for the fused path.
 """
 import math
@@ -17,8 +17,7 @@ import math
 import torch
 import torch.nn as nn
 
-from omni_moe.ops.hip import (hip_linear_func, hip_omni_expert_func, hip_omni_mlp_func, hip_omni_moe_fwd_func,
-                              hip_omni_router_fwd_func, hip_omni_router_func)
+from omni_moe.ops.hip import hip_omni_expert_func, hip_omni_mlp_func, hip_omni_moe_fwd_func, hip_omni_router_fwd_func
 
 
 class OmniMoEConfig:
@@ -104,12 +103,7 @@ class OmniMoE(nn.Module):
         """The reference's composition (omni_moe.py:64-104) over the differentiable operators."""
         bsz, seq_len, _ = hidden_states.shape
         x = hidden_states.reshape(-1, self.hidden_size)
-        logits_x = self.router_norm_x(hip_linear_func(x, self.router_gate_x.weight))
-        logits_y = self.router_norm_y(hip_linear_func(x, self.router_gate_y.weight))
-        logits_x = torch.nn.functional.log_softmax(logits_x, dim=-1)
-        logits_y = torch.nn.functional.log_softmax(logits_y, dim=-1)
-        scores, indices = hip_omni_router_func(logits_x, logits_y, self.num_expert_sqrt, self.top_k)
-        routing_weights = torch.exp(scores)
+        routing_weights, indices = self.route(x)          # one differentiable node (OmniRouterStageFunc)
         experts_states = hip_omni_expert_func(x, self.up_embed.weight, self.down_embed.weight, routing_weights, indices)
         mlp_states = hip_omni_mlp_func(x, self.gate_proj.weight, self.up_proj.weight, self.down_proj.weight)
         return (mlp_states + experts_states).view(bsz, seq_len, -1)

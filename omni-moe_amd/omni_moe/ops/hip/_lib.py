@@ -48,6 +48,9 @@ SIGNATURES = {
     "omni_expert_bwd": (c_int32, [c_void_p] * 10 + [c_int64, c_int32, c_int64, c_int32, c_int32, c_void_p, c_void_p]),
     "omni_swiglu_fwd": (c_int32, [c_void_p] * 3 + [c_int64, c_int32, c_void_p]),
     "omni_swiglu_bwd": (c_int32, [c_void_p] * 5 + [c_int64, c_int32, c_void_p]),
+    "omni_router_workspace_stats_offset": (c_size_t, [c_int64, c_int32, c_int32]),
+    "omni_router_norm_bwd_workspace_bytes": (c_size_t, [c_int64, c_int32]),
+    "omni_router_norm_bwd": (c_int32, [c_void_p] * 6 + [c_int64, c_int32, c_int32, c_int32, c_int32, c_void_p, c_void_p]),
 }
 
 _lib = None

@@ -434,8 +434,23 @@ def hip_omni_router_fwd_func(
     for nbt in (num_batches_tracked_x, num_batches_tracked_y):
         if nbt is not None and (nbt.dtype != torch.int64 or nbt.numel() != 1):
             raise TypeError("num_batches_tracked must be an int64 scalar tensor")
-    dev = _lib.require_gpu(x, weight_x, weight_y, *stats)
-    x, weight_x, weight_y = map(_c, (x, weight_x, weight_y))
+    _lib.require_gpu(x, weight_x, weight_y, *stats)
+    if _needs_grad(x, weight_x, weight_y):
+        if return_scores:
+            raise ValueError("the differentiable router stage returns gates and indices only")
+        return OmniRouterStageFunc.apply(x, weight_x, weight_y, running_mean_x, running_var_x, num_batches_tracked_x,
+                                         running_mean_y, running_var_y, num_batches_tracked_y, k, bool(training),
+                                         float(momentum), float(eps))
+    out = _router_stage_forward(x, weight_x, weight_y, running_mean_x, running_var_x, num_batches_tracked_x,
+                                running_mean_y, running_var_y, num_batches_tracked_y, k, training, momentum, eps, return_scores)
+    return out[:3] if return_scores else out[:2]
+
+
+def _router_stage_forward(x, weight_x, weight_y, running_mean_x, running_var_x, num_batches_tracked_x,
+                          running_mean_y, running_var_y, num_batches_tracked_y, k, training, momentum, eps, return_scores=False):
+    """(gates, indices, scores or None, workspace): the workspace still holds z and the BatchNorm statistics."""
+    x, weight_x, weight_y = (_c(t.detach()) for t in (x, weight_x, weight_y))
+    dev, r = x.device, weight_x.size(0)
     T, H = x.shape
     lib = _lib.load()
     dt = _lib.DTYPE_CODE[x.dtype]
@@ -451,7 +466,50 @@ def hip_omni_router_fwd_func(
             1 if training else 0, float(momentum), float(eps), _lib.ptr(gates), _lib.ptr(indices), _lib.ptr(scores),
             T, H, r, k, dt, _lib.DTYPE_CODE[running_mean_x.dtype], _lib.ptr(ws), _lib.stream_ptr())
     _lib.check(code, "omni_router_fwd")
-    return (gates, indices, scores) if return_scores else (gates, indices)
+    return gates, indices, scores, ws
+
+
+def hip_omni_router_stage_bwd_func(dgates, gates, indices, workspace, num_tokens, num_expert_sqrt, training):
+    """d(z) [T, 2r] of the router stage from d(gates), using z and the statistics that ``omni_router_fwd`` left in
+    ``workspace`` (exp, router op, log_softmax and BatchNorm1d of reference omni_moe.py:70-86 in reverse)."""
+    lib = _lib.load()
+    dev = _lib.require_gpu(dgates, gates, indices, workspace)
+    T, r, k = int(num_tokens), int(num_expert_sqrt), gates.size(1)
+    dt = _lib.DTYPE_CODE[gates.dtype]
+    dgates = _c(dgates)
+    off = lib.omni_router_workspace_stats_offset(T, r, dt)
+    dz = torch.empty((T, 2 * r), device=dev, dtype=gates.dtype)
+    ws = torch.empty(max(lib.omni_router_norm_bwd_workspace_bytes(T, r), 1), device=dev, dtype=torch.uint8)
+    with torch.cuda.device(dev):
+        code = lib.omni_router_norm_bwd(_lib.ptr(dgates), _lib.ptr(gates), _lib.ptr(indices), workspace.data_ptr(),
+                                        workspace.data_ptr() + off, _lib.ptr(dz), T, r, k, dt, 1 if training else 0,
+                                        _lib.ptr(ws), _lib.stream_ptr())
+    _lib.check(code, "omni_router_norm_bwd")
+    return dz
+
+
+class OmniRouterStageFunc(torch.autograd.Function):
+    """The layer's router (projection, BatchNorm1d, log_softmax, router op, exp; reference omni_moe.py:70-86) as one
+    differentiable node: the forward is ``omni_router_fwd``, the backward one HIP pass from d(gates) to d(z) and the two
+    library GEMMs for d(weights) and d(x)."""
+
+    @staticmethod
+    def forward(ctx, x, weight_x, weight_y, rmx, rvx, nbtx, rmy, rvy, nbty, k, training, momentum, eps):
+        gates, indices, _, ws = _router_stage_forward(x, weight_x, weight_y, rmx, rvx, nbtx, rmy, rvy, nbty, k, training,
+                                                      momentum, eps)
+        ctx.save_for_backward(x, weight_x, weight_y, gates, indices, ws)
+        ctx.training = training
+        ctx.mark_non_differentiable(indices)
+        return gates, indices
+
+    @staticmethod
+    def backward(ctx, dgates, _dindices):
+        x, weight_x, weight_y, gates, indices, ws = ctx.saved_tensors
+        r = weight_x.size(0)
+        dz = hip_omni_router_stage_bwd_func(dgates, gates, indices, ws, x.size(0), r, ctx.training)
+        dw = dz.t().matmul(x) if (ctx.needs_input_grad[1] or ctx.needs_input_grad[2]) else None
+        dx = dz.matmul(torch.cat([weight_x, weight_y])) if ctx.needs_input_grad[0] else None
+        return (dx, dw[:r] if dw is not None else None, dw[r:] if dw is not None else None) + (None,) * 10
 
 
 def hip_omni_moe_fwd_func(

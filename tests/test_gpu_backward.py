@@ -297,3 +297,49 @@ def test_backward_edge_cases(device):
         hip.hip_omni_router_bwd_func(torch.randn(4, 2, device=device), torch.zeros(4, 3, dtype=torch.int32, device=device), 8)
     with pytest.raises(ValueError):                                   # r beyond what the kernel covers
         hip.hip_omni_router_bwd_func(torch.randn(4, 2, device=device), torch.zeros(4, 2, dtype=torch.int32, device=device), 2048)
+
+
+@pytest.mark.parametrize("training", [True, False], ids=["train", "eval"])
+@pytest.mark.parametrize("case", [(256, 128, 32, 8), (300, 64, 7, 6), (100, 96, 100, 16), (64, 64, 300, 32)],
+                         ids=lambda c: f"T{c[0]}-H{c[1]}-r{c[2]}-k{c[3]}")
+def test_router_stage_backward_matches_autograd(case, training, device):
+    """OmniRouterStageFunc (projection, BatchNorm1d, log_softmax, router op, exp as one node) in fp32: gates and
+    the gradients of x and both router weights against fp64 autograd of the same composition, evaluated at the
+    ids the GPU selected."""
+    T, H, r, k = case
+    g = torch.Generator().manual_seed(T + r)
+    x = torch.randn(T, H, generator=g)
+    wx, wy = torch.randn(r, H, generator=g) * 0.2, torch.randn(r, H, generator=g) * 0.2
+    run_mean, run_var = torch.randn(2, r, generator=g) * 0.1, torch.rand(2, r, generator=g) + 0.5
+    w = torch.randn(T, k, generator=g)
+    hip = _ops()
+    leaves = [t.to(device).requires_grad_() for t in (x, wx, wy)]
+    bufs = [t.to(device).clone() for t in (run_mean[0], run_var[0], run_mean[1], run_var[1])]
+    nbt = [torch.zeros((), dtype=torch.long, device=device) for _ in range(2)]
+    print(f"router stage T={T} H={H} r={r} k={k} training={training}", flush=True)
+    gates, ids = hip.hip_omni_router_fwd_func(leaves[0], leaves[1], leaves[2], bufs[0], bufs[1], nbt[0], bufs[2], bufs[3], nbt[1],
+                                              k, training=training)
+    assert gates.requires_grad and not ids.requires_grad
+    (gates * w.to(device)).sum().backward()
+
+    cx, cwx, cwy = (t.double().requires_grad_() for t in (x, wx, wy))
+
+    def half(weight, mean, var):
+        z = cx @ weight.t()
+        if training:
+            z = (z - z.mean(0)) / torch.sqrt(z.var(0, unbiased=False) + 1e-5)
+        else:
+            z = (z - mean.double()) / torch.sqrt(var.double() + 1e-5)
+        return torch.log_softmax(z, -1)
+
+    lx, ly = half(cwx, run_mean[0], run_var[0]), half(cwy, run_mean[1], run_var[1])
+    scores = (lx.unsqueeze(2) + ly.unsqueeze(1)).reshape(T, r * r).gather(1, ids.cpu().long())
+    want = torch.exp(scores)
+    (want * w.double()).sum().backward()
+    _close(gates.detach(), want.detach(), torch.float32, "gates")
+    for leaf, c, what in zip(leaves, (cx, cwx, cwy), ("dx", "dweight_x", "dweight_y")):
+        assert torch.isfinite(leaf.grad).all()
+        err = (leaf.grad.double().cpu() - c.grad).abs().max().item() / max(c.grad.abs().max().item(), 1e-30)
+        assert err <= 2e-4, f"{what}: max error {err:.3e}"
+    if training:
+        assert nbt[0].item() == 1 and nbt[1].item() == 1
