@@ -353,3 +353,26 @@ def test_layer_is_graph_capturable(overlap, device):
         assert torch.equal(y, want)
         assert torch.equal(layer(x * 0.5), layer(x * 0.5))      # eager work between the replays
         torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("training", [True, False], ids=["train", "eval"])
+@pytest.mark.parametrize("T", [1, 2, 3, 5, 31, 33, 65])
+def test_layer_tiny_token_counts(T, training, device):
+    """A handful of tokens (one wave, one partial strip, a single BatchNorm sample in training), on one and on two
+    streams: same tolerance as the big cases, and both schedules bit-identical."""
+    from omni_moe.modules.omni_moe import OmniMoE, OmniMoEConfig
+    H, I, N, k = 128, 256, 256, 8
+    x, w = oracle.make_layer_inputs(T, T, H, I, N)
+    sd = {"gate_proj.weight": w.gate_proj, "up_proj.weight": w.up_proj, "down_proj.weight": w.down_proj,
+          "router_gate_x.weight": w.router_gate_x, "router_gate_y.weight": w.router_gate_y,
+          "up_embed.weight": w.up_embed, "down_embed.weight": w.down_embed}
+    want, _, _ = oracle.moe_forward(x, w, oracle.BNState.fresh(16), oracle.BNState.fresh(16), k, training)
+    outs = []
+    for overlap in (True, False):
+        layer = OmniMoE(OmniMoEConfig(H, I, "silu", N, k))
+        layer.load_state_dict(sd, strict=False)
+        layer = layer.to(device=device, dtype=torch.bfloat16).train(training)
+        layer.overlap_branches = overlap
+        outs.append(layer(x.to(device)))
+    torch.testing.assert_close(outs[0].cpu().float(), want.float(), rtol=2e-2, atol=2e-2)
+    assert torch.equal(outs[0], outs[1])
