@@ -75,6 +75,29 @@ __device__ __forceinline__ float wave_max(float v) {
   return v;
 }
 
+// Value of lane (lane ^ STRIDE) without touching LDS memory: DPP quad permutes (1, 2), two
+// bank-masked DPP row shifts (4, 8), a ds_swizzle bit pattern (16), v_permlane32_swap (32).
+template <int STRIDE>
+__device__ __forceinline__ int xor_lane_i(int v, int lane) {
+  if constexpr (STRIDE == 1) return __builtin_amdgcn_update_dpp(v, v, 0xB1, 0xf, 0xf, false);
+  else if constexpr (STRIDE == 2) return __builtin_amdgcn_update_dpp(v, v, 0x4E, 0xf, 0xf, false);
+  else if constexpr (STRIDE == 4) {
+    const int t = __builtin_amdgcn_update_dpp(v, v, 0x104, 0xf, 0x5, false);     // row_shl:4 into banks 0,2
+    return __builtin_amdgcn_update_dpp(t, v, 0x114, 0xf, 0xA, false);            // row_shr:4 into banks 1,3
+  } else if constexpr (STRIDE == 8) {
+    const int t = __builtin_amdgcn_update_dpp(v, v, 0x108, 0xf, 0x3, false);     // row_shl:8 into banks 0,1
+    return __builtin_amdgcn_update_dpp(t, v, 0x118, 0xf, 0xC, false);            // row_shr:8 into banks 2,3
+  } else if constexpr (STRIDE == 16) return __builtin_amdgcn_ds_swizzle(v, 0x401F);
+  else {
+    const auto sw = __builtin_amdgcn_permlane32_swap(v, v, false, false);         // [lo,lo] and [hi,hi]
+    return (lane & 32) ? (int)sw[0] : (int)sw[1];
+  }
+}
+template <int STRIDE>
+__device__ __forceinline__ float xor_lane_f(float v, int lane) {
+  return __int_as_float(xor_lane_i<STRIDE>(__float_as_int(v), lane));
+}
+
 // x*sigmoid(x) in fp32, IEEE division.
 __device__ __forceinline__ float silu_f32(float x) { return x / (1.0f + __expf(-x)); }
 // Same with the hardware reciprocal (1 ulp) and exp2: ~6 instructions.  For results that are

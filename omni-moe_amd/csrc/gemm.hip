@@ -100,9 +100,27 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, f32x16_t (&acc)
                                               const int wm, const int wn, const int lane) {
   constexpr int TNO = (EPI == kEpiSwiglu) ? TN / 2 : TN;
   // ---- column statistics of the rounded tile for BatchNorm: every 32-row MFMA tile is one
-  // strip; a column lives in the 32 lanes that share lane/32, so five xor-shuffles reduce it
+  // strip.  A column's 32 rows sit in the 32 lanes that share lane/32, one of this lane's 16
+  // values each, so the 16 columns of a half-wave are reduced together: a butterfly that halves
+  // the values a lane keeps at every step (8 + 4 + 2 + 1 + 1 exchanges) leaves each lane pair
+  // with the sum of ONE column; the means travel back the same way (1 + 2 + 4 + 8), the squared
+  // deviations are reduced like the sums.  47 register-to-register exchanges per tile.
   if constexpr (EPI == kEpiStats) {
     if (g.part_mean) {
+      const bool b16 = lane & 16, b8 = lane & 8, b4 = lane & 4, b2 = lane & 2;
+      auto reduce_scatter = [&](const float (&v)[16]) -> float {
+        float a8[8], a4[4], a2[2];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) a8[e] = (b16 ? v[e + 8] : v[e]) + xor_lane_f<16>(b16 ? v[e] : v[e + 8], lane);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) a4[e] = (b8 ? a8[e + 4] : a8[e]) + xor_lane_f<8>(b8 ? a8[e] : a8[e + 4], lane);
+#pragma unroll
+        for (int e = 0; e < 2; ++e) a2[e] = (b4 ? a4[e + 2] : a4[e]) + xor_lane_f<4>(b4 ? a4[e] : a4[e + 2], lane);
+        const float a1 = (b2 ? a2[1] : a2[0]) + xor_lane_f<2>(b2 ? a2[0] : a2[1], lane);
+        return a1 + xor_lane_f<1>(a1, lane);
+      };
+      // the column this lane ends up with: q = 8*b16 + 4*b8 + 2*b4 + b2
+      const int q_mine = (b16 ? 8 : 0) + (b8 ? 4 : 0) + (b4 ? 2 : 0) + (b2 ? 1 : 0);
 #pragma unroll
       for (int i = 0; i < TM; ++i) {
         const int row0 = m0 + wm * TM * 32 + i * 32;
@@ -110,23 +128,46 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, f32x16_t (&acc)
         if (cnt <= 0) continue;
         const bool live = (lane & 31) < cnt;
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
+        for (int j = 0; j < TN; ++j) {
+          float v[16];
 #pragma unroll
-          for (int q = 0; q < 16; ++q) {
-            const float v = live ? Elem<DT>::round(acc[i][j][q]) : 0.f;
-            float sum = v;
-#pragma unroll
-            for (int mk = 16; mk >= 1; mk >>= 1) sum += __shfl_xor(sum, mk, kWave);
-            const float mean = sum / float(cnt);
-            float dev = live ? (v - mean) * (v - mean) : 0.f;
-#pragma unroll
-            for (int mk = 16; mk >= 1; mk >>= 1) dev += __shfl_xor(dev, mk, kWave);
-            const int n = n0 + wn * TN * 32 + j * 32 + (q >> 2) * 8 + (lane >> 5) * 4 + (q & 3);
-            if ((lane & 31) == 0 && n < g.N) {
-              g.part_mean[(int64_t)(row0 >> 5) * g.N + n] = mean;
-              g.part_m2[(int64_t)(row0 >> 5) * g.N + n] = dev;
-            }
+          for (int q = 0; q < 16; ++q) v[q] = live ? Elem<DT>::round(acc[i][j][q]) : 0.f;
+          const float mean = reduce_scatter(v) / float(cnt);
+          // all-gather of the 16 means, index = column
+          float g2[2], g4[4], g8[8], mu[16];
+          {
+            const float o = xor_lane_f<2>(mean, lane);
+            g2[0] = b2 ? o : mean;
+            g2[1] = b2 ? mean : o;
           }
+#pragma unroll
+          for (int e = 0; e < 2; ++e) {
+            const float o = xor_lane_f<4>(g2[e], lane);
+            g4[e] = b4 ? o : g2[e];
+            g4[e + 2] = b4 ? g2[e] : o;
+          }
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const float o = xor_lane_f<8>(g4[e], lane);
+            g8[e] = b8 ? o : g4[e];
+            g8[e + 4] = b8 ? g4[e] : o;
+          }
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const float o = xor_lane_f<16>(g8[e], lane);
+            mu[e] = b16 ? o : g8[e];
+            mu[e + 8] = b16 ? g8[e] : o;
+          }
+          float d[16];
+#pragma unroll
+          for (int q = 0; q < 16; ++q) d[q] = live ? (v[q] - mu[q]) * (v[q] - mu[q]) : 0.f;
+          const float m2 = reduce_scatter(d);
+          const int n = n0 + wn * TN * 32 + j * 32 + (q_mine >> 2) * 8 + (lane >> 5) * 4 + (q_mine & 3);
+          if ((lane & 1) == 0 && n < g.N) {
+            g.part_mean[(int64_t)(row0 >> 5) * g.N + n] = mean;
+            g.part_m2[(int64_t)(row0 >> 5) * g.N + n] = m2;
+          }
+        }
       }
     }
   }
@@ -592,8 +633,8 @@ static int gemm_plain(const void* a, const void* b, const void* b_hi, const void
     else if (mid >= 200) err = launch_gemm<DT, 2, 2, kEpiResidual>(g, s);
     else err = launch_gemm<DT, 1, 1, kEpiResidual>(g, s);
   } else if (part_mean) {
-    // the statistics keep every accumulator live through a long reduction: 128 x 128 tiles at most
-    if (mid >= 200) err = launch_gemm<DT, 2, 2, kEpiStats>(g, s);
+    if (big >= 200) err = launch_gemm<DT, 4, 4, kEpiStats>(g, s);
+    else if (mid >= 200) err = launch_gemm<DT, 2, 2, kEpiStats>(g, s);
     else err = launch_gemm<DT, 1, 1, kEpiStats>(g, s);
   } else {
     if (big >= 200) err = launch_gemm<DT, 4, 4, kEpiPlain>(g, s);

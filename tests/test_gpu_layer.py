@@ -65,7 +65,9 @@ def test_mlp_fp32_matches_oracle(case, device):
     torch.testing.assert_close(got_r, want + res, rtol=1e-4, atol=1e-5 * max(1.0, want.abs().max().item()))
 
 
-ROUTER_FWD_CASES = [(4096, 1024, 64, 16), (1024, 256, 32, 8), (2048, 2048, 512, 32), (300, 520, 36, 10)]
+# the last two make the projection GEMM pick its 128 x 128 and 256 x 256 tiles (statistics epilogue included)
+ROUTER_FWD_CASES = [(4096, 1024, 64, 16), (1024, 256, 32, 8), (2048, 2048, 512, 32), (300, 520, 36, 10),
+                    (4096, 256, 512, 32), (16384, 256, 512, 32)]
 
 
 def _bn_buffers(r, dtype, device=None):
