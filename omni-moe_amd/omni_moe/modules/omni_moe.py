@@ -86,6 +86,9 @@ class OmniMoE(nn.Module):
     # kernel (cache bandwidth, no LDS) shares CUs with the projections (LDS and MFMA).  Set to False
     # to keep everything on one stream, with the add as the down projection's epilogue.
     overlap_branches = True
+    # The fork and join cost about 50 us of host time per call, so below this much work (tokens x hidden x
+    # intermediate; 2048 x 1024 x 4096 measured level on an MI355X) the call would be host-bound: one stream then.
+    overlap_min_work = 2 ** 33
 
     def _branch_resources(self, device):
         res = self.__dict__.get("_omni_branch")
@@ -117,7 +120,9 @@ class OmniMoE(nn.Module):
             raise NotImplementedError("cumulative-average BatchNorm (momentum=None) is not covered")
         with torch.no_grad():
             x = hidden_states.view(-1, self.hidden_size)
-            side, fork, join = self._branch_resources(x.device) if (self.overlap_branches and x.is_cuda) else (None, None, None)
+            two = (self.overlap_branches and x.is_cuda
+                   and x.size(0) * self.hidden_size * self.intermediate_size > self.overlap_min_work)
+            side, fork, join = self._branch_resources(x.device) if two else (None, None, None)
             out = hip_omni_moe_fwd_func(
                 x, self.gate_proj.weight, self.up_proj.weight, self.down_proj.weight,
                 self.router_gate_x.weight, self.router_gate_y.weight,

@@ -277,6 +277,7 @@ def test_layer_two_streams_equals_one_stream(dtype, device):
     from omni_moe.modules.omni_moe import OmniMoE, OmniMoEConfig
     torch.manual_seed(0)
     layer = OmniMoE(OmniMoEConfig(256, 512, "silu", 1024, 8)).to(device=device, dtype=dtype).eval()
+    layer.overlap_min_work = 0                    # two streams whatever the size
     x = torch.randn(3, 100, 256, device=device).to(dtype)
     layer.overlap_branches = False
     ref = layer(x)
@@ -338,6 +339,7 @@ def test_layer_is_graph_capturable(overlap, device):
     torch.manual_seed(1)
     layer = OmniMoE(OmniMoEConfig(256, 512, "silu", 1024, 8)).to(device=device, dtype=torch.bfloat16).eval()
     layer.overlap_branches = overlap
+    layer.overlap_min_work = 0
     x = torch.randn(2, 150, 256, device=device).bfloat16()
     want = layer(x).clone()
     warm = torch.cuda.Stream()
@@ -375,6 +377,7 @@ def test_layer_tiny_token_counts(T, training, device):
         layer.load_state_dict(sd, strict=False)
         layer = layer.to(device=device, dtype=torch.bfloat16).train(training)
         layer.overlap_branches = overlap
+        layer.overlap_min_work = 0
         outs.append(layer(x.to(device)))
     torch.testing.assert_close(outs[0].cpu().float(), want.float(), rtol=2e-2, atol=2e-2)
     assert torch.equal(outs[0], outs[1])
