@@ -28,8 +28,12 @@ for p in (os.path.join(ROOT, "omni-moe_amd"), ROOT):
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 # Fabric-side bytes per launch (FETCH_SIZE + WRITE_SIZE, each scaled by a plain copy of known size) from the
 # rocprofv3 --pmc runs summarised in profiles/bench_layer_c4_hbm_counters.txt; counters cannot be read in-process.
-TRAFFIC_BYTES = {"expert_c3": 897.5e6, "expert_c4": 224.9e6, "gateup_c4": 134.7e6, "down_c4": 117.6e6}
+TRAFFIC_BYTES = {"expert_c3": 184.0e6, "expert_c4": 57.8e6, "expert_gather_c3": 897.8e6, "gateup_c4": 134.7e6, "down_c4": 117.6e6}
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
+
+
+EXPERT_NOTE = ("the 16 MiB up/down tables are served from the caches (each XCD's L2 holds the eighth of them its blocks use), "
+               "so algorithmic bytes exceed fabric traffic and the fraction of HBM peak exceeds 1")
 
 
 def expert_alg_bytes(T, H, k, s=2):
@@ -170,8 +174,8 @@ def main():
         kernels = [
             mfma_entry("gemm_nt_dma_kernel<swiglu> (gate/up projection + SwiGLU), c4", 4 * T * H * I, ms_gateup, TRAFFIC_BYTES["gateup_c4"]),
             mfma_entry("gemm_nt_dma_kernel<residual> (down projection + experts add), c4", 2 * T * H * I, ms_down, TRAFFIC_BYTES["down_c4"]),
-            hbm_entry("expert_gather_kernel, c4", expert_alg_bytes(T, H, k), ms_expert,
-                      "up/down tables (16 MiB) are cache-resident, so algorithmic bytes exceed HBM traffic", TRAFFIC_BYTES["expert_c4"]),
+            hbm_entry("expert op (split algorithm: expert_split_dots_kernel + expert_split_accumulate_kernel), c4", expert_alg_bytes(T, H, k),
+                      ms_expert, EXPERT_NOTE, TRAFFIC_BYTES["expert_c4"]),
             {"kernel": "router stage (projection GEMM with BN statistics epilogue + BN finalize + select), c4", "kernel_ms": ms_router,
              "algorithmic_flops": 4 * T * H * r},
         ]
@@ -179,16 +183,19 @@ def main():
         T3 = 16384
         x3, up3, down3, g3, i3 = (t.to(dev) for t in oracle.make_expert_inputs(2, T3, H, N, k))
         ms_e3 = time_call(torch, lambda: hip.hip_omni_expert_func(x3, up3, down3, g3, i3), reps)
+        ms_g3 = time_call(torch, lambda: hip.hip_omni_expert_func(x3, up3, down3, g3, i3, algo="gather"), reps)
         ms_s3 = time_call(torch, lambda: hip.hip_omni_schedule_func(i3, N), reps)
         ms_seg3 = time_call(torch, lambda: hip.hip_omni_expert_func(x3, up3, down3, g3, i3, algo="segment"), reps)
-        kernels.append(hbm_entry("expert_gather_kernel, c3 (T=16384)", expert_alg_bytes(T3, H, k), ms_e3,
-                                 "up/down tables (16 MiB) are cache-resident, so algorithmic bytes exceed HBM traffic",
-                                 TRAFFIC_BYTES["expert_c3"]))
+        kernels.append(hbm_entry("expert op (split algorithm: expert_split_dots_kernel + expert_split_accumulate_kernel), c3 (T=16384)",
+                                 expert_alg_bytes(T3, H, k), ms_e3, EXPERT_NOTE, TRAFFIC_BYTES["expert_c3"]))
+        kernels.append(hbm_entry("expert op, gather algorithm (expert_gather_kernel), c3", expert_alg_bytes(T3, H, k), ms_g3,
+                                 "for comparison: whole rows per wave, three quarters of them fetched over the fabric",
+                                 TRAFFIC_BYTES["expert_gather_c3"]))
         kernels.append(hbm_entry("schedule (stable counting sort: count, scan x2, scatter, offsets), c3", T3 * k * 14 + 8 * (N + 1), ms_s3))
         kernels.append(hbm_entry("expert op, expert-centric 'segment' algorithm (schedule + scores pass + token pass), c3",
-                                 expert_alg_bytes(T3, H, k), ms_seg3, "for comparison with expert_gather_kernel; same results"))
+                                 expert_alg_bytes(T3, H, k), ms_seg3, "for comparison; same results as the gather algorithm"))
         out["roofline"] = max(kernels[:3], key=lambda d: d["kernel_ms"])
-        out["roofline_expert"] = kernels[-3]
+        out["roofline_expert"] = kernels[-4]
         # training path (not part of the forward metric): backward of the expert op at the same shape
         dy3 = x3 * 0.5
         ms_b3 = time_call(torch, lambda: hip.hip_omni_expert_bwd_func(dy3, x3, up3, down3, g3, i3), reps)

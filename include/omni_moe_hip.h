@@ -50,6 +50,7 @@ extern "C" {
 #define OMNI_EXPERT_ALGO_AUTO 0
 #define OMNI_EXPERT_ALGO_GATHER 1   /* token-resident gather, no schedule needed */
 #define OMNI_EXPERT_ALGO_SEGMENT 2  /* expert-centric segments from omni_schedule */
+#define OMNI_EXPERT_ALGO_SPLIT 3    /* hidden dimension cut into 8 slices, one per XCD: table slices stay in that XCD's L2 */
 
 OMNI_API int32_t omni_abi_version(void);
 OMNI_API const char* omni_error_string(int32_t code);
@@ -91,10 +92,16 @@ OMNI_API int32_t omni_schedule(const int32_t* indices, int32_t* offsets, int32_t
  *   indices [T,k] int32 in [0,N) (duplicates inside a token add; not range-checked,
  *   as in the reference); y [T,H] dtype `dtype`, fully overwritten.
  * H*sizeof(elem) must be a multiple of 16.  Sums are fp32, one rounding at the end.
- *   algo      : OMNI_EXPERT_ALGO_* (AUTO = GATHER).  SEGMENT is the expert-centric organisation:
+ *   algo      : OMNI_EXPERT_ALGO_*.  GATHER: one wave per token fetches whole rows.  SPLIT: the hidden
+ *               dimension in 8 slices, slice s handled by the blocks that run on XCD s, so that
+ *               each XCD's L2 holds its eighth of both tables; two launches and [8][T][k] floats
+ *               of partial dot products (H*sizeof(elem)/8 must be 64..1024 bytes, a power of two).
+ *               AUTO = SPLIT when the tables overflow one L2 but an eighth of them fits and there
+ *               are >= 32768 pairs, else GATHER.  SEGMENT is the expert-centric organisation:
  *               omni_schedule, a pass over the sorted pairs for the coefficients, a token pass
- *               for the sum; same results, kept so that both can be measured.
- *   workspace : omni_expert_workspace_bytes() bytes (0 for GATHER: may be NULL) */
+ *               for the sum; kept so that the organisations can be measured side by side.
+ *               GATHER and SEGMENT agree bit for bit, SPLIT to fp32 rounding of the dot products.
+ *   workspace : omni_expert_workspace_bytes() bytes for the same arguments (0 = may be NULL) */
 OMNI_API size_t omni_expert_workspace_bytes(int64_t num_tokens, int32_t hidden_size, int64_t num_experts,
                                    int32_t num_experts_per_token, int32_t dtype, int32_t algo);
 OMNI_API int32_t omni_expert_fwd(const void* x, const void* up_weight, const void* down_weight,

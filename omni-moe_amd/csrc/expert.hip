@@ -266,13 +266,190 @@ static int expert_segment_dispatch(const void* x, const void* up, const void* do
   return err == hipSuccess ? OMNI_OK : OMNI_ERR_HIP_BASE + (int)err;
 }
 
+// ---- hidden-split variant ("split" algorithm) ------------------------------------------------
+// For tables that fit the chip's caches but not one XCD's 4 MiB L2 (16 MiB at N = 4096,
+// H = 1024): the hidden dimension is cut into 8 slices and slice s is only ever touched by
+// blocks with blockIdx % 8 == s, which the dispatcher places on XCD s.  An XCD then needs
+// N * H/8 elements of each table -- 1 MiB each in that example -- and serves every table row
+// from its own L2 instead of pulling three quarters of them over the fabric.  The price is a
+// cross-slice reduction of the pair scores, which is tiny ([8][T][k] floats):
+//   A. block (token group, slice): partial dot products <x[t, slice], up[id, slice]> for the k pairs
+//      of each of its tokens -> partial[slice][t][j];
+//   B. block (token group, slice): coefficient silu(sum over slices, in slice order) * gate, then
+//      y[t, slice] = sum_j coefficient_j * down[id_j, slice].
+// A row slice is LPR lanes of 16 bytes (64 / LPR pairs per wave at a time).  Fixed summation
+// order, no atomics; results agree with the gather algorithm to fp32 rounding of the dot product.
+constexpr int kSlices = 8;
+
+// Sum over the LPR lanes of a group of LPR values per lane, scattered: lane `sub` of the group
+// ends up with the total of value `sub`.  Every step halves what a lane keeps (LPR - 1 exchanges
+// in all, against LPR * log2(LPR) for one tree per value).
+template <int LPR, int N = LPR>
+__device__ __forceinline__ float reduce_scatter_group(float (&v)[N], const int lane) {
+  if constexpr (N == 1) {
+    return v[0];
+  } else {
+    constexpr int S = N / 2;                   // lane distance of this step = half of what is left
+    const bool upper = lane & S;
+    float keep[S];
+#pragma unroll
+    for (int e = 0; e < S; ++e) keep[e] = (upper ? v[e + S] : v[e]) + xor_lane_f<S>(upper ? v[e] : v[e + S], lane);
+    return reduce_scatter_group<LPR, S>(keep, lane);
+  }
+}
+
+// A wave owns GP = 64 / LPR tokens, one per lane group; the group's LPR lanes cover the token's
+// row slice, 16 bytes each.  Pairs go in batches of LPR: LPR partial dot products per lane,
+// then one reduce-scatter leaves pair `sub` of the batch in lane `sub`.
+template <int DT, int LPR>
+__global__ __launch_bounds__(kTokensPerBlock* kWave) void expert_split_dots_kernel(
+    const uint8_t* __restrict__ x, const uint8_t* __restrict__ up, const int32_t* __restrict__ ids,
+    float* __restrict__ partial, int num_tokens, int hidden, int top_k, uint32_t num_experts) {
+  constexpr int E = Row16<DT>::kElems, GP = kWave / LPR;
+  constexpr int LD = LPR < 8 ? LPR : 8;                          // row loads in flight at a time
+  const int lane = lane_id(), sub = lane % LPR, grp = lane / LPR;
+  const int slice = blockIdx.x % kSlices;
+  const int t = ((int)(blockIdx.x / kSlices) * kTokensPerBlock + (threadIdx.x >> 6)) * GP + grp;
+  const bool live = t < num_tokens;
+  const int tt = live ? t : 0;
+  const int64_t row_bytes = int64_t(hidden) * (16 / E);
+  const int64_t col = int64_t(slice) * LPR * 16 + sub * 16;      // this lane's 16 bytes inside a row
+  const u32x4_t xr = *(const u32x4_t*)(x + tt * row_bytes + col);
+  const int64_t base = int64_t(tt) * top_k;
+  for (int jb = 0; jb < top_k; jb += LPR) {
+    float d[LPR];
+#pragma unroll
+    for (int e0 = 0; e0 < LPR; e0 += LD) {
+      u32x4_t ur[LD];
+#pragma unroll
+      for (int e = 0; e < LD; ++e) {
+        const int j = min(jb + e0 + e, top_k - 1);
+        const int id = ids[base + j];                            // one address per group: a broadcast load
+        ur[e] = *(const u32x4_t*)(up + int64_t((uint32_t)id < num_experts ? id : 0) * row_bytes + col);
+      }
+#pragma unroll
+      for (int e = 0; e < LD; ++e) d[e0 + e] = dot16<DT>(xr, ur[e], 0.f);
+    }
+    const float total = reduce_scatter_group<LPR>(d, lane);
+    const int j = jb + sub;
+    if (live && j < top_k) {
+      const bool ok = (uint32_t)ids[base + j] < num_experts;
+      partial[(int64_t(slice) * num_tokens + t) * top_k + j] = ok ? total : 0.f;
+    }
+  }
+}
+
+// Same ownership.  Lane `sub` of a group forms the coefficient of pair `sub` of a batch (sum of
+// the 8 slice partials in slice order, silu, gate); the group then walks the batch, every lane
+// fetching its 16 bytes of the down row and the pair's coefficient from the lane that holds it.
+template <int DT, int LPR>
+__global__ __launch_bounds__(kTokensPerBlock* kWave) void expert_split_accumulate_kernel(
+    const uint8_t* __restrict__ down, const void* __restrict__ gates, const int32_t* __restrict__ ids,
+    const float* __restrict__ partial, uint8_t* __restrict__ y, int num_tokens, int hidden, int top_k, uint32_t num_experts) {
+  constexpr int E = Row16<DT>::kElems, GP = kWave / LPR;
+  constexpr int LD = LPR < 8 ? LPR : 8;
+  const int lane = lane_id(), sub = lane % LPR, grp = lane / LPR;
+  const int slice = blockIdx.x % kSlices;
+  const int t = ((int)(blockIdx.x / kSlices) * kTokensPerBlock + (threadIdx.x >> 6)) * GP + grp;
+  const bool live = t < num_tokens;
+  const int tt = live ? t : 0;
+  const int64_t row_bytes = int64_t(hidden) * (16 / E);
+  const int64_t col = int64_t(slice) * LPR * 16 + sub * 16;
+  const int64_t base = int64_t(tt) * top_k;
+  float acc[E];
+#pragma unroll
+  for (int i = 0; i < E; ++i) acc[i] = 0.f;
+  for (int jb = 0; jb < top_k; jb += LPR) {
+    const int j = jb + sub;
+    float coef = 0.f;
+    int my_id = 0;
+    if (j < top_k) {
+      float sdot = 0.f;
+#pragma unroll
+      for (int sl = 0; sl < kSlices; ++sl) sdot += partial[(int64_t(sl) * num_tokens + tt) * top_k + j];
+      const int id = ids[base + j];
+      if ((uint32_t)id < num_experts) {
+        my_id = id;
+        coef = silu_f32(sdot) * Elem<DT>::load(gates, base + j);
+      }
+    }
+#pragma unroll
+    for (int e0 = 0; e0 < LPR; e0 += LD) {
+      u32x4_t vr[LD];
+      float cf[LD];
+#pragma unroll
+      for (int e = 0; e < LD; ++e) {
+        const int src = grp * LPR + e0 + e;                       // the lane of this group that holds pair e0+e
+        cf[e] = __shfl(coef, src, kWave);
+        vr[e] = *(const u32x4_t*)(down + int64_t(__shfl(my_id, src, kWave)) * row_bytes + col);
+      }
+#pragma unroll
+      for (int e = 0; e < LD; ++e) axpy16<DT>(cf[e], vr[e], acc);
+    }
+  }
+  if (live) *(u32x4_t*)(y + t * row_bytes + col) = pack16<DT>(acc);
+}
+
+// lanes per row slice, or 0 when the row does not cut into 8 slices of 4..64 lanes
+static inline int split_lanes_per_row(int hidden, int elem_bytes) {
+  const int64_t slice_bytes = (int64_t)hidden * elem_bytes / kSlices;
+  if ((int64_t)hidden * elem_bytes % (kSlices * 16) != 0) return 0;
+  const int lpr = (int)(slice_bytes / 16);
+  return (lpr == 4 || lpr == 8 || lpr == 16 || lpr == 32 || lpr == 64) ? lpr : 0;
+}
+
+template <int DT, int LPR>
+static hipError_t launch_split(const void* x, const void* up, const void* down, const void* gates, const int32_t* ids,
+                               float* partial, void* y, int64_t T, int H, int k, int64_t N, hipStream_t s) {
+  constexpr int kPerBlock = kTokensPerBlock * (kWave / LPR);       // tokens per block
+  const unsigned blocks = (unsigned)((T + kPerBlock - 1) / kPerBlock) * kSlices;
+  hipLaunchKernelGGL((expert_split_dots_kernel<DT, LPR>), dim3(blocks), dim3(kTokensPerBlock * kWave), 0, s, (const uint8_t*)x,
+                     (const uint8_t*)up, ids, partial, (int)T, H, k, (uint32_t)N);
+  hipLaunchKernelGGL((expert_split_accumulate_kernel<DT, LPR>), dim3(blocks), dim3(kTokensPerBlock * kWave), 0, s,
+                     (const uint8_t*)down, gates, ids, partial, (uint8_t*)y, (int)T, H, k, (uint32_t)N);
+  return hipGetLastError();
+}
+
+// workspace: partial dot products [8][T][k] f32
+template <int DT>
+static int expert_split_dispatch(const void* x, const void* up, const void* down, const void* gates, const int32_t* ids,
+                                 void* y, int64_t T, int H, int k, int64_t N, void* workspace, hipStream_t s) {
+  const int lpr = split_lanes_per_row(H, DT == kF32 ? 4 : 2);
+  if (lpr == 0 || k > 2 * kWave) return OMNI_ERR_UNSUPPORTED;
+  if (T == 0) return OMNI_OK;
+  if (k == 0) return expert_gather_dispatch<DT>(x, up, down, gates, ids, y, T, H, k, N, s);   // writes zeros
+  if (!workspace) return OMNI_ERR_WORKSPACE;
+  float* partial = (float*)workspace;
+  hipError_t err;
+  if (lpr == 4) err = launch_split<DT, 4>(x, up, down, gates, ids, partial, y, T, H, k, N, s);
+  else if (lpr == 8) err = launch_split<DT, 8>(x, up, down, gates, ids, partial, y, T, H, k, N, s);
+  else if (lpr == 16) err = launch_split<DT, 16>(x, up, down, gates, ids, partial, y, T, H, k, N, s);
+  else if (lpr == 32) err = launch_split<DT, 32>(x, up, down, gates, ids, partial, y, T, H, k, N, s);
+  else err = launch_split<DT, 64>(x, up, down, gates, ids, partial, y, T, H, k, N, s);
+  return err == hipSuccess ? OMNI_OK : OMNI_ERR_HIP_BASE + (int)err;
+}
+
+// What OMNI_EXPERT_ALGO_AUTO runs.  The split algorithm pays when the two tables overflow one
+// XCD's 4 MiB L2 while an eighth of them fits beside the streaming x and y rows, and when there
+// are enough pairs to amortise its second launch; otherwise rows are gathered whole.
+static int resolve_algo(int algo, int64_t T, int H, int64_t N, int k, int dtype) {
+  if (algo != OMNI_EXPERT_ALGO_AUTO) return algo;
+  const int es = dtype == OMNI_F32 ? 4 : 2;
+  const int64_t tables = 2 * N * (int64_t)H * es;
+  const bool fits = split_lanes_per_row(H, es) != 0 && k <= 2 * kWave;
+  if (fits && tables > (3ll << 20) && tables / kSlices <= (3ll << 20) && T * (int64_t)k >= 32768) return OMNI_EXPERT_ALGO_SPLIT;
+  return OMNI_EXPERT_ALGO_GATHER;
+}
+
 }  // namespace omni
 
 extern "C" OMNI_API size_t omni_expert_workspace_bytes(int64_t num_tokens, int32_t hidden_size, int64_t num_experts,
                                                        int32_t num_experts_per_token, int32_t dtype, int32_t algo) {
-  (void)hidden_size; (void)dtype;
-  if (algo != OMNI_EXPERT_ALGO_SEGMENT) return 0;   // the gather algorithm keeps everything in registers
   if (num_tokens < 0 || num_experts <= 0 || num_experts_per_token < 0) return 0;
+  algo = omni::resolve_algo(algo, num_tokens, hidden_size, num_experts, num_experts_per_token, dtype);
+  if (algo == OMNI_EXPERT_ALGO_SPLIT)
+    return omni::align256((size_t)omni::kSlices * (size_t)num_tokens * (size_t)num_experts_per_token * 4);
+  if (algo != OMNI_EXPERT_ALGO_SEGMENT) return 0;   // the gather algorithm keeps everything in registers
   const size_t P = (size_t)num_tokens * (size_t)num_experts_per_token;
   return omni::align256((size_t)(num_experts + 1) * 4) + 2 * omni::align256(P * 4) +
          omni_schedule_workspace_bytes(num_tokens, num_experts_per_token, num_experts);
@@ -289,6 +466,7 @@ extern "C" OMNI_API int32_t omni_expert_fwd(const void* x, const void* up_weight
   if (num_tokens > 0 && (!x || !up_weight || !down_weight || !y)) return OMNI_ERR_NULL;
   if (num_tokens > 0 && num_experts_per_token > 0 && (!routing_weights || !indices)) return OMNI_ERR_NULL;
   hipStream_t s = (hipStream_t)stream;
+  algo = resolve_algo(algo, num_tokens, hidden_size, num_experts, num_experts_per_token, dtype);
   if (algo == OMNI_EXPERT_ALGO_SEGMENT) {
     switch (dtype) {
       case OMNI_BF16: return expert_segment_dispatch<kBF16>(x, up_weight, down_weight, routing_weights, indices, y, num_tokens, hidden_size, num_experts_per_token, num_experts, workspace, s);
@@ -297,7 +475,15 @@ extern "C" OMNI_API int32_t omni_expert_fwd(const void* x, const void* up_weight
       default: return OMNI_ERR_DTYPE;
     }
   }
-  if (algo != OMNI_EXPERT_ALGO_AUTO && algo != OMNI_EXPERT_ALGO_GATHER) return OMNI_ERR_UNSUPPORTED;
+  if (algo == OMNI_EXPERT_ALGO_SPLIT) {
+    switch (dtype) {
+      case OMNI_BF16: return expert_split_dispatch<kBF16>(x, up_weight, down_weight, routing_weights, indices, y, num_tokens, hidden_size, num_experts_per_token, num_experts, workspace, s);
+      case OMNI_F16: return expert_split_dispatch<kF16>(x, up_weight, down_weight, routing_weights, indices, y, num_tokens, hidden_size, num_experts_per_token, num_experts, workspace, s);
+      case OMNI_F32: return expert_split_dispatch<kF32>(x, up_weight, down_weight, routing_weights, indices, y, num_tokens, hidden_size, num_experts_per_token, num_experts, workspace, s);
+      default: return OMNI_ERR_DTYPE;
+    }
+  }
+  if (algo != OMNI_EXPERT_ALGO_GATHER) return OMNI_ERR_UNSUPPORTED;
   switch (dtype) {
     case OMNI_BF16: return expert_gather_dispatch<kBF16>(x, up_weight, down_weight, routing_weights, indices, y, num_tokens, hidden_size, num_experts_per_token, num_experts, s);
     case OMNI_F16: return expert_gather_dispatch<kF16>(x, up_weight, down_weight, routing_weights, indices, y, num_tokens, hidden_size, num_experts_per_token, num_experts, s);

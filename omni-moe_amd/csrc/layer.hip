@@ -11,16 +11,17 @@ static inline size_t up256(size_t v) { return (v + 255) / 256 * 256; }
 static inline size_t elem_bytes(int dtype) { return dtype == OMNI_F32 ? 4 : 2; }
 }  // namespace omni
 
-// workspace: router workspace | gates [T,k] | ids [T,k] | expert output [T,H] | SwiGLU activations [T,I]
+// workspace: router workspace | gates [T,k] | ids [T,k] | expert output [T,H] | expert workspace | SwiGLU activations [T,I]
 extern "C" OMNI_API size_t omni_moe_workspace_bytes(int64_t num_tokens, int32_t hidden_size, int32_t intermediate_size,
                                                     int64_t num_experts, int32_t num_expert_sqrt, int32_t num_experts_per_token,
                                                     int32_t dtype) {
   using namespace omni;
-  (void)num_experts;
   if (num_tokens < 0 || hidden_size <= 0 || intermediate_size <= 0 || num_expert_sqrt <= 0 || num_experts_per_token < 0) return 0;
   const size_t es = elem_bytes(dtype), T = (size_t)num_tokens, k = (size_t)num_experts_per_token;
   return up256(omni_router_workspace_bytes(num_tokens, num_expert_sqrt, dtype)) + up256(T * k * es) + up256(T * k * 4) +
-         up256(T * (size_t)hidden_size * es) + up256(omni_mlp_workspace_bytes(num_tokens, hidden_size, intermediate_size, dtype));
+         up256(T * (size_t)hidden_size * es) +
+         up256(omni_expert_workspace_bytes(num_tokens, hidden_size, num_experts, num_experts_per_token, dtype, OMNI_EXPERT_ALGO_AUTO)) +
+         up256(omni_mlp_workspace_bytes(num_tokens, hidden_size, intermediate_size, dtype));
 }
 
 extern "C" OMNI_API int32_t omni_moe_fwd(const void* x, const void* gate_weight, const void* up_weight, const void* down_weight,
@@ -53,6 +54,8 @@ extern "C" OMNI_API int32_t omni_moe_fwd(const void* x, const void* gate_weight,
   void* gates = w;      w += up256(T * k * es);
   int32_t* ids = (int32_t*)w;  w += up256(T * k * 4);
   void* experts = w;    w += up256(T * (size_t)hidden_size * es);
+  void* expert_ws = w;
+  w += up256(omni_expert_workspace_bytes(num_tokens, hidden_size, num_experts, num_experts_per_token, dtype, OMNI_EXPERT_ALGO_AUTO));
   void* h = w;
 
   hipStream_t main_s = (hipStream_t)stream;
@@ -69,7 +72,7 @@ extern "C" OMNI_API int32_t omni_moe_fwd(const void* x, const void* gate_weight,
     return e;
   if ((e = omni_swiglu_linear_fwd(x, gate_weight, up_weight, h, num_tokens, hidden_size, intermediate_size, dtype, main_s))) return e;
   if ((e = omni_expert_fwd(x, up_embed, down_embed, gates, ids, experts, num_tokens, hidden_size, num_experts,
-                           num_experts_per_token, dtype, OMNI_EXPERT_ALGO_GATHER, nullptr, branch)))
+                           num_experts_per_token, dtype, OMNI_EXPERT_ALGO_AUTO, expert_ws, branch)))
     return e;
   if (!side_stream)   // one stream: the add is the down projection's epilogue
     return omni_linear_fwd(h, down_weight, experts, y, num_tokens, intermediate_size, hidden_size, dtype, main_s);

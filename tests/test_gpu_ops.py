@@ -181,6 +181,50 @@ def test_expert_segment_algorithm_equals_gather(case, device):
     assert torch.equal(a, b)
 
 
+def _split_covers(H, dtype):
+    slice_bytes = H * torch.empty((), dtype=dtype).element_size() // 8
+    return H * torch.empty((), dtype=dtype).element_size() % 128 == 0 and slice_bytes in (64, 128, 256, 512, 1024)
+
+
+@pytest.mark.parametrize("case", EXPERT_CASES + [(4100, 1024, 4096, 16, torch.bfloat16, "ref"), (1000, 256, 512, 10, torch.float16, "ref"),
+                                                 (130, 512, 64, 34, torch.float32, "ref"), (64, 4096, 16, 128, torch.bfloat16, "ref")],
+                         ids=lambda c: f"T{c[0]}-H{c[1]}-N{c[2]}-k{c[3]}-{str(c[4]).split('.')[-1]}-{c[5]}")
+def test_expert_split_algorithm(case, device):
+    """The hidden-split organisation (8 column slices, one per XCD, partial dot products summed in slice order):
+    same tolerance against the oracle, agreement with the gather algorithm to fp32 rounding, run-to-run identical;
+    rows that do not cut into 8 power-of-two slices are refused."""
+    T, H, N, k, dtype, kind = case
+    x, up, down, gates, ids = _expert_inputs(T, H, N, k, dtype, kind, seed=T + H)
+    d = [t.to(device) for t in (x, up, down, gates, ids)]
+    print(f"expert split T={T} H={H} N={N} k={k} {dtype} {kind}", flush=True)
+    if not _split_covers(H, dtype):
+        with pytest.raises(ValueError):
+            _ops().hip_omni_expert_func(*d, algo="split")
+        return
+    got = _ops().hip_omni_expert_func(*d, algo="split")
+    assert torch.equal(got, _ops().hip_omni_expert_func(*d, algo="split"))
+    want = oracle.expert_forward(x, up, down, gates, ids)
+    torch.testing.assert_close(got.cpu().float(), want.float(), **_tol(dtype))
+    ref = _ops().hip_omni_expert_func(*d, algo="gather").float()
+    scale = max(ref.abs().max().item(), 1e-6)
+    # one storage ulp at most where the fp32 sums straddle a rounding boundary
+    assert (got.float() - ref).abs().max().item() <= (1e-2 if dtype != torch.float32 else 1e-5) * scale
+
+
+def test_expert_split_bad_ids(device):
+    g = torch.Generator().manual_seed(12)
+    T, H, N, k = 2100, 1024, 512, 8
+    x, up, down = torch.randn(T, H, generator=g).bfloat16(), (torch.randn(N, H, generator=g) * 0.05).bfloat16(), (torch.randn(N, H, generator=g) * 0.05).bfloat16()
+    gates = torch.rand(T, k, generator=g).bfloat16()
+    ids = torch.randint(0, N, (T, k), generator=g, dtype=torch.int32)
+    ids[::7, 3] = N + 5
+    ids[::11, 0] = -1
+    ok = (ids >= 0) & (ids < N)
+    want = oracle.expert_forward(x, up, down, torch.where(ok, gates, torch.zeros_like(gates)), torch.where(ok, ids, torch.zeros_like(ids)))
+    got = _ops().hip_omni_expert_func(*(t.to(device) for t in (x, up, down, gates, ids)), algo="split")
+    torch.testing.assert_close(got.cpu().float(), want.float(), rtol=2e-2, atol=2e-2)
+
+
 def test_expert_segment_skewed_and_bad_ids(device):
     g = torch.Generator().manual_seed(11)
     T, H, N, k = 4096, 1024, 512, 8
