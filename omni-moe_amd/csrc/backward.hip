@@ -299,8 +299,10 @@ __global__ __launch_bounds__(kBwdWavesPerBlock* kWave, 2) void expert_bwd_token_
         ds_out[base + j0 + i] = ds;
         coef_out[base + j0 + i] = coef;
       }
+      if (live_slot[i]) {                       // not even 0 * row: the stand-in row may hold Inf or NaN
 #pragma unroll
-      for (int c = 0; c < NCH; ++c) axpy16<DT>(ds, ur[i][c], acc[c]);
+        for (int c = 0; c < NCH; ++c) axpy16<DT>(ds, ur[i][c], acc[c]);
+      }
     }
   }
 #pragma unroll

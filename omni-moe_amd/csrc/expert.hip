@@ -96,7 +96,8 @@ __global__ __launch_bounds__(kTokensPerBlock* kWave, 2) void expert_gather_kerne
     for (int i = 0; i < G; ++i) s[i] = wave_sum(s[i]);
 #pragma unroll
     for (int i = 0; i < G; ++i) {
-      const float coef = live_slot[i] ? silu_f32(s[i]) * g[i] : 0.f;
+      if (!live_slot[i]) continue;                  // not even 0 * row: the stand-in row may hold Inf or NaN
+      const float coef = silu_f32(s[i]) * g[i];
 #pragma unroll
       for (int c = 0; c < NCH; ++c) axpy16<DT>(coef, vr[i][c], acc[c]);
     }
@@ -204,12 +205,14 @@ __global__ __launch_bounds__(kTokensPerBlock* kWave, 2) void expert_accumulate_k
   }
   for (int j0 = 0; j0 < top_k; j0 += G) {
     float cf[G];
+    bool used[G];
     u32x4_t vr[G][NCH];
 #pragma unroll
     for (int i = 0; i < G; ++i) {
       const int j = min(j0 + i, top_k - 1);
       const int id = ids[int64_t(t) * top_k + j];
       const bool ok = (j0 + i < top_k) && (uint32_t)id < num_experts;
+      used[i] = ok;
       cf[i] = ok ? coef[int64_t(t) * top_k + j] : 0.f;
       const int e = ok ? id : 0;
 #pragma unroll
@@ -217,9 +220,11 @@ __global__ __launch_bounds__(kTokensPerBlock* kWave, 2) void expert_accumulate_k
         vr[i][c] = live[c] ? *(const u32x4_t*)(down + e * row_bytes + off[c]) : u32x4_t{0, 0, 0, 0};
     }
 #pragma unroll
-    for (int i = 0; i < G; ++i)
+    for (int i = 0; i < G; ++i) {
+      if (!used[i]) continue;
 #pragma unroll
       for (int c = 0; c < NCH; ++c) axpy16<DT>(cf[i], vr[i][c], acc[c]);
+    }
   }
 #pragma unroll
   for (int c = 0; c < NCH; ++c)
@@ -362,7 +367,7 @@ __global__ __launch_bounds__(kTokensPerBlock* kWave) void expert_split_accumulat
   for (int jb = 0; jb < top_k; jb += LPR) {
     const int j = jb + sub;
     float coef = 0.f;
-    int my_id = 0;
+    int my_id = -1;                                               // -1: a padded slot or an id outside the table
     if (j < top_k) {
       float sdot = 0.f;
 #pragma unroll
@@ -377,14 +382,18 @@ __global__ __launch_bounds__(kTokensPerBlock* kWave) void expert_split_accumulat
     for (int e0 = 0; e0 < LPR; e0 += LD) {
       u32x4_t vr[LD];
       float cf[LD];
+      bool used[LD];
 #pragma unroll
       for (int e = 0; e < LD; ++e) {
         const int src = grp * LPR + e0 + e;                       // the lane of this group that holds pair e0+e
+        const int id = __shfl(my_id, src, kWave);
         cf[e] = __shfl(coef, src, kWave);
-        vr[e] = *(const u32x4_t*)(down + int64_t(__shfl(my_id, src, kWave)) * row_bytes + col);
+        used[e] = id >= 0;
+        vr[e] = *(const u32x4_t*)(down + int64_t(used[e] ? id : 0) * row_bytes + col);
       }
 #pragma unroll
-      for (int e = 0; e < LD; ++e) axpy16<DT>(cf[e], vr[e], acc);
+      for (int e = 0; e < LD; ++e)
+        if (used[e]) axpy16<DT>(cf[e], vr[e], acc);             // not even 0 * row: the stand-in row may hold Inf or NaN
     }
   }
   if (live) *(u32x4_t*)(y + t * row_bytes + col) = pack16<DT>(acc);

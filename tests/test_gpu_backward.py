@@ -343,3 +343,19 @@ def test_router_stage_backward_matches_autograd(case, training, device):
         assert err <= 2e-4, f"{what}: max error {err:.3e}"
     if training:
         assert nbt[0].item() == 1 and nbt[1].item() == 1
+
+
+def test_expert_bwd_unused_rows_may_hold_nan(device):
+    """As in the forward: the row that stands in for padded slots and out-of-range ids must not leak into any gradient."""
+    T, H, N, k = 300, 256, 64, 6
+    x, up, down, gates, ids = oracle.make_expert_inputs(14, T, H, N, k, dtype=torch.float32, w_std=0.05)
+    ids = ids.clamp(min=1)
+    ids[::9, 2] = N + 1
+    dy = torch.randn(T, H, generator=torch.Generator().manual_seed(3))
+    d = [t.to(device) for t in (dy, x, up, down, gates, ids)]
+    want = _ops().hip_omni_expert_bwd_func(*d)
+    up2, down2 = up.clone(), down.clone()
+    up2[0], down2[0] = float("nan"), float("inf")
+    got = _ops().hip_omni_expert_bwd_func(d[0], d[1], up2.to(device), down2.to(device), d[4], d[5])
+    for a, b in zip(got, want):
+        assert torch.isfinite(a).all() and torch.equal(a, b)

@@ -274,3 +274,19 @@ def test_schedule_drops_out_of_range_ids(device):
     order = torch.sort(torch.where(valid, flat, torch.full_like(flat, N)).long(), stable=True).indices
     assert torch.equal(pairs[:nv], order[:nv])
     assert torch.equal(torch.sort(pairs).values, torch.arange(T * k))       # still a permutation
+
+
+@pytest.mark.parametrize("algo", ["gather", "segment", "split"])
+def test_expert_unused_rows_may_hold_nan(algo, device):
+    """Padded slots and ids outside the table stand in for row 0 when rows are fetched; whatever row 0 holds must not
+    leak: with NaN in the rows of experts that no valid pair selects, every output stays finite and unchanged."""
+    T, H, N, k = 2100, 256, 2048, 6                                # k is no multiple of any batch size
+    x, up, down, gates, ids = _expert_inputs(T, H, N, k, torch.bfloat16, "ref", seed=5)
+    ids = ids.clamp(min=1)                                         # nobody selects expert 0 ...
+    ids[::9, 2] = N + 1                                            # ... and some ids fall outside the table
+    d = [t.to(device) for t in (x, up, down, gates, ids)]
+    want = _ops().hip_omni_expert_func(*d, algo=algo)
+    up2, down2 = up.clone(), down.clone()
+    up2[0], down2[0] = float("nan"), float("inf")
+    got = _ops().hip_omni_expert_func(d[0], up2.to(device), down2.to(device), d[3], d[4], algo=algo)
+    assert torch.isfinite(got).all() and torch.equal(got, want)
