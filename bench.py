@@ -28,7 +28,7 @@ for p in (os.path.join(ROOT, "omni-moe_amd"), ROOT):
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 # Fabric-side bytes per launch (FETCH_SIZE + WRITE_SIZE, each scaled by a plain copy of known size) from the
 # rocprofv3 --pmc runs summarised in profiles/bench_layer_c4_hbm_counters.txt; counters cannot be read in-process.
-TRAFFIC_BYTES = {"expert_c3": 184.0e6, "expert_c4": 57.8e6, "expert_gather_c3": 897.8e6, "gateup_c4": 134.7e6, "down_c4": 117.6e6}
+TRAFFIC_BYTES = {"expert_c3": 183.2e6, "expert_c4": 57.8e6, "expert_gather_c3": 897.9e6, "gateup_c4": 134.7e6, "down_c4": 117.6e6}
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 
 
