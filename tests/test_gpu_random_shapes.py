@@ -93,3 +93,35 @@ def test_expert_and_linear_random_shapes(device):
         ref = x.double() @ up.double().t()
         ulp = {torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -11, torch.float32: 2.0 ** -22}[dtype]
         assert ((y.double() - ref).abs() <= ulp * ref.abs() * 1.01 + 1e-4 * max(ref.abs().max().item(), 1e-6)).all(), case
+
+
+def test_layer_random_shapes_fp32(device):
+    """Whole layer in fp32 (where near-ties in the router are rare), train and eval, one and two streams."""
+    from omni_moe.modules.omni_moe import OmniMoE, OmniMoEConfig
+    rng = random.Random(5)
+    for case in range(12):
+        H = 4 * rng.choice([4, 8, 9, 16, 33, 64])
+        I = 4 * rng.choice([4, 8, 16, 17, 64])
+        N = rng.choice([4, 9, 50, 64, 100, 257, 1024])
+        r = int(N ** 0.5)
+        k = 2 * rng.randint(1, max(1, min(8, r * r // 2)))
+        T = rng.choice([1, 5, 64, 200, 777])
+        training = rng.random() < 0.5
+        x, w = oracle.make_layer_inputs(100 + case, T, H, I, N, dtype=torch.float32, w_std=0.1)
+        sd = {"gate_proj.weight": w.gate_proj, "up_proj.weight": w.up_proj, "down_proj.weight": w.down_proj,
+              "router_gate_x.weight": w.router_gate_x, "router_gate_y.weight": w.router_gate_y,
+              "up_embed.weight": w.up_embed, "down_embed.weight": w.down_embed}
+        print(f"layer case {case}: T={T} H={H} I={I} N={N} r={r} k={k} training={training}", flush=True)
+        want, _, want_i = oracle.moe_forward(x, w, oracle.BNState.fresh(r), oracle.BNState.fresh(r), k, training)
+        outs = []
+        for overlap in (True, False):
+            layer = OmniMoE(OmniMoEConfig(H, I, "silu", N, k))
+            layer.load_state_dict(sd, strict=False)
+            layer = layer.to(device).train(training)
+            layer.overlap_branches, layer.overlap_min_work = overlap, 0
+            with torch.no_grad():
+                outs.append(layer(x.to(device)))
+        assert torch.equal(outs[0], outs[1]), case
+        scale = max(want.abs().max().item(), 1e-6)
+        err = (outs[0].cpu() - want).abs().max().item()
+        assert err <= 2e-4 * scale, (case, err, scale)
