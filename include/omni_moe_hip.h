@@ -44,6 +44,7 @@ extern "C" {
 #define OMNI_ERR_TOPK (-4)        /* num_experts_per_token violates the router contract */
 #define OMNI_ERR_UNSUPPORTED (-5) /* valid request that no kernel here covers */
 #define OMNI_ERR_WORKSPACE (-6)   /* workspace NULL or too small */
+#define OMNI_ERR_SCRATCH (-7)     /* request exceeds the fixed device scratch of omni_schedule_noalloc */
 #define OMNI_ERR_HIP_BASE 1000    /* + hipError_t */
 
 /* expert algorithms */
@@ -84,6 +85,19 @@ OMNI_API size_t omni_schedule_workspace_bytes(int64_t num_tokens, int32_t num_ex
 OMNI_API int32_t omni_schedule(const int32_t* indices, int32_t* offsets, int32_t* sorted_pair_ids,
                       int32_t* sorted_token_ids, int64_t num_tokens, int32_t num_experts_per_token,
                       int64_t num_experts, void* workspace, void* stream);
+
+/* omni_schedule for callers that cannot allocate: code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc.  No counterpart in the reference.  Same arguments and results as
+ * omni_schedule, without the workspace: the sort's scratch is a fixed array of
+ * OMNI_SCHEDULE_NOALLOC_SCRATCH_BYTES that every GPU the library runs on holds until the process ends.
+ * The call allocates and frees nothing.  Requests whose omni_schedule_workspace_bytes() exceeds the
+ * array return OMNI_ERR_SCRATCH (nothing enqueued); 262 144 pairs over 4096 experts fit.
+ * All calls on one GPU share that GPU's array: calls that may overlap on the device (different
+ * streams without an ordering between them) race; calls on one stream are safe. */
+#define OMNI_SCHEDULE_NOALLOC_SCRATCH_BYTES (8u << 20)
+OMNI_API int32_t omni_schedule_noalloc(const int32_t* indices, int32_t* offsets, int32_t* sorted_pair_ids,
+                              int32_t* sorted_token_ids, int64_t num_tokens, int32_t num_experts_per_token,
+                              int64_t num_experts, void* stream);
 
 /* Fused atomic-expert forward  y[t] = sum_j silu(<x[t],U[id_tj]>) * g_tj * V[id_tj].
  * Replaces triton_omni_expert_func / omni_expert_forward

@@ -12,6 +12,7 @@ extern "C" OMNI_API const char* omni_error_string(int32_t code) {
     case OMNI_ERR_TOPK: return "num_experts_per_token must be even, <= 128 and <= num_expert_sqrt^2";
     case OMNI_ERR_UNSUPPORTED: return "valid request that no kernel of this library covers";
     case OMNI_ERR_WORKSPACE: return "workspace is NULL or too small";
+    case OMNI_ERR_SCRATCH: return "the request needs more than the fixed device scratch of the entry point that allocates nothing";
     default: return code >= OMNI_ERR_HIP_BASE ? "the HIP runtime refused a launch (code - 1000 is the hipError_t)" : "unknown error code";
   }
 }

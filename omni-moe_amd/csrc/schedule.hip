@@ -294,3 +294,50 @@ extern "C" OMNI_API int32_t omni_schedule(const int32_t* indices, int32_t* offse
   hipError_t err = hipGetLastError();
   return err == hipSuccess ? OMNI_OK : OMNI_ERR_HIP_BASE + (int)err;
 }
+
+// ---- the same schedule for callers that cannot allocate ---------------------------------------
+// Code under HIP graph capture, tight serving loops and harnesses that forbid hipMalloc have no
+// way to bring a workspace.  For them the sort's workspace is a fixed array in device memory that
+// each GPU holds from the moment the library is loaded until the process ends.  In host code the
+// array's name is only a handle: its device address is looked up once per device with
+// hipGetSymbolAddress and kept; every kernel receives that address as its workspace argument.
+namespace omni {
+
+static __device__ __align__(256) unsigned char scratch[OMNI_SCHEDULE_NOALLOC_SCRATCH_BYTES];
+
+constexpr int kMaxDevices = 64;
+static std::atomic<void*> g_scratch_addr[kMaxDevices];
+
+// Device address of `scratch` on the current device (resolved on the first call per device).
+static int scratch_address(void** out) {
+  int dev = -1;
+  if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return OMNI_ERR_HIP_BASE + (int)e;
+  if (dev < 0 || dev >= kMaxDevices) return OMNI_ERR_UNSUPPORTED;
+  void* p = g_scratch_addr[dev].load(std::memory_order_acquire);
+  if (!p) {
+    if (hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)); e != hipSuccess) return OMNI_ERR_HIP_BASE + (int)e;
+    if (!p) return OMNI_ERR_SCRATCH;
+    g_scratch_addr[dev].store(p, std::memory_order_release);   // concurrent first calls store the same address
+  }
+  *out = p;
+  return OMNI_OK;
+}
+
+}  // namespace omni
+
+extern "C" OMNI_API int32_t omni_schedule_noalloc(const int32_t* indices, int32_t* offsets, int32_t* sorted_pair_ids,
+                                                  int32_t* sorted_token_ids, int64_t num_tokens, int32_t num_experts_per_token,
+                                                  int64_t num_experts, void* stream) {
+  using namespace omni;
+  const int64_t N = num_experts, P = num_tokens * (int64_t)num_experts_per_token;
+  if (num_tokens < 0 || num_experts_per_token < 0 || N <= 0 || P > INT32_MAX / 2 || N > INT32_MAX / 2) return OMNI_ERR_SHAPE;
+  SortPlan pl;
+  if (!make_plan(P, N, &pl)) return OMNI_ERR_UNSUPPORTED;
+  const size_t need = omni_schedule_workspace_bytes(num_tokens, num_experts_per_token, num_experts);
+  if (need == 0 || need > (size_t)OMNI_SCHEDULE_NOALLOC_SCRATCH_BYTES) return OMNI_ERR_SCRATCH;
+  void* ws = nullptr;
+  if (int e = scratch_address(&ws)) return e;
+  // every kernel of the sort writes the part of the workspace it later reads (counts, tile sums,
+  // keys, pair ids), so nothing of an earlier call's contents has to be cleared
+  return omni_schedule(indices, offsets, sorted_pair_ids, sorted_token_ids, num_tokens, num_experts_per_token, num_experts, ws, stream);
+}

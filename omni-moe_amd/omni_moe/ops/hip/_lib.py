@@ -29,6 +29,7 @@ SIGNATURES = {
     "omni_router_select": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int32, c_int32, c_int32, c_void_p]),
     "omni_schedule_workspace_bytes": (c_size_t, [c_int64, c_int32, c_int64]),
     "omni_schedule": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int32, c_int64, c_void_p, c_void_p]),
+    "omni_schedule_noalloc": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int32, c_int64, c_void_p]),
     "omni_expert_workspace_bytes": (c_size_t, [c_int64, c_int32, c_int64, c_int32, c_int32, c_int32]),
     "omni_mlp_workspace_bytes": (c_size_t, [c_int64, c_int32, c_int32, c_int32]),
     "omni_mlp_fwd": (c_int32, [c_void_p] * 6 + [c_int64, c_int32, c_int32, c_int32, c_void_p, c_void_p]),

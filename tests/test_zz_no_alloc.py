@@ -1,0 +1,60 @@
+"""omni_schedule_noalloc (the entry point that allocates nothing) against omni_schedule, through the C ABI."""
+import pytest
+import torch
+
+from omni_moe.ops.hip import _lib
+
+pytestmark = pytest.mark.gpu
+
+
+def _both(idx: torch.Tensor, N: int):
+    lib = _lib.load()
+    T, k = idx.shape
+    dev = idx.device
+
+    def outputs():
+        return (torch.full((N + 1,), -1, device=dev, dtype=torch.int32), torch.full((T * k,), -1, device=dev, dtype=torch.int32),
+                torch.full((T * k,), -1, device=dev, dtype=torch.int32))
+
+    want, got = outputs(), outputs()
+    ws = torch.empty(max(lib.omni_schedule_workspace_bytes(T, k, N), 1), device=dev, dtype=torch.uint8)
+    stream = _lib.stream_ptr()
+    _lib.check(lib.omni_schedule(_lib.ptr(idx), *(t.data_ptr() for t in want), T, k, N, _lib.ptr(ws), stream), "omni_schedule")
+    before = torch.cuda.memory_allocated(dev)
+    code = lib.omni_schedule_noalloc(_lib.ptr(idx), *(t.data_ptr() for t in got), T, k, N, stream)
+    assert torch.cuda.memory_allocated(dev) == before
+    _lib.check(code, "omni_schedule_noalloc")
+    torch.cuda.synchronize(dev)
+    return want, got
+
+
+def test_noalloc_schedule_equals_schedule_twice_in_a_row(device):
+    g = torch.Generator().manual_seed(11)
+    N = 4096
+    big = torch.randint(0, N, (16384, 16), generator=g, dtype=torch.int32)
+    big[5, 3] = -7                      # ids outside [0, N) go behind the last segment in both entry points
+    big[9, 0] = N + 2
+    small = torch.randint(0, 100, (300, 6), generator=g, dtype=torch.int32)
+    for idx, n in ((big, N), (small, 100)):          # the second call is smaller and finds the first one's leftovers
+        want, got = _both(idx.to(device), n)
+        for w, h, name in zip(want, got, ("offsets", "sorted_pair_ids", "sorted_token_ids")):
+            assert torch.equal(w, h), name
+        off = want[0].cpu()
+        cnt = torch.bincount(idx.flatten()[(idx.flatten() >= 0) & (idx.flatten() < n)].long(), minlength=n)
+        assert torch.equal(off[1:] - off[:-1], cnt.int())
+
+
+def test_noalloc_schedule_two_pass_sort_and_limit(device):
+    lib = _lib.load()
+    g = torch.Generator().manual_seed(12)
+    N = 262144                           # two counting passes
+    idx = torch.randint(0, N, (2048, 32), generator=g, dtype=torch.int32).to(device)
+    want, got = _both(idx, N)
+    for w, h in zip(want, got):
+        assert torch.equal(w, h)
+    # beyond the fixed scratch: a clear error, nothing enqueued
+    T, k = 1 << 20, 16
+    assert lib.omni_schedule_workspace_bytes(T, k, 4096) > (8 << 20)
+    p = idx.data_ptr()
+    assert lib.omni_schedule_noalloc(p, p, p, p, T, k, 4096, _lib.stream_ptr()) == -7
+    assert b"scratch" in lib.omni_error_string(-7)
