@@ -14,6 +14,8 @@
 #include "common.h"
 #include "omni_moe_hip.h"
 
+#include <type_traits>
+
 namespace omni {
 
 #ifdef OMNI_GEMM_TIMING
@@ -423,9 +425,6 @@ __global__ __launch_bounds__(kGemmThreads, 1) void gemm_nt_dma_kernel(const Gemm
   const int wm = wave & 1, wn = wave >> 1;
   int tile_m, tile_n;
   tile_coords(g, tile_m, tile_n);
-#ifdef OMNI_GEMM_SAME_TILE
-  tile_m &= 1; tile_n &= 1;   // debug: every block works on one of 4 tiles (operands stay in L2)
-#endif
   const int m0 = tile_m * BM, n0 = tile_n * BN;
 
   // load instruction p of wave w fills tile rows (4p+w)*kRpi ..: lane -> row lane/kCpr, position lane%kCpr
@@ -460,25 +459,20 @@ __global__ __launch_bounds__(kGemmThreads, 1) void gemm_nt_dma_kernel(const Gemm
   }
 
   const int wave_s = __builtin_amdgcn_readfirstlane(wave);   // scalar copy: LDS destinations stay in SGPRs
-  // one quarter (part 0..3) of a tile's LPT load instructions; parts are spread between MFMA
-  // groups so that their address set-up and issue never leave the matrix pipeline idle
-  auto issue_part = [&](int kt, int part) {
+  // load instruction q (0 .. LPT-1) of tile kt: first the PA instructions of the activation tile, then the weights'
+  auto issue_one = [&](int kt, int q) __attribute__((always_inline)) {
     uint8_t* st = lds + (kt % NS) * kStageBytes;
     const int koff = kt * kRow;
-#pragma unroll
-    for (int q = 0; q < LPT; ++q) {
-      if ((q * 4) / LPT != part) continue;
-      if (q < PA)
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(a_src[q] + koff),
-                                         (__attribute__((address_space(3))) void*)(st + (4 * q + wave_s) * 1024), 16, 0, 0);
-      else
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(b_src[q - PA] + koff),
-                                         (__attribute__((address_space(3))) void*)(st + BM * kRow + (4 * (q - PA) + wave_s) * 1024), 16, 0, 0);
-    }
+    if (q < PA)
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(a_src[q] + koff),
+                                       (__attribute__((address_space(3))) void*)(st + (4 * q + wave_s) * 1024), 16, 0, 0);
+    else
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(b_src[q - PA] + koff),
+                                       (__attribute__((address_space(3))) void*)(st + BM * kRow + (4 * (q - PA) + wave_s) * 1024), 16, 0, 0);
   };
   auto issue_tile = [&](int kt) {
 #pragma unroll
-    for (int part = 0; part < 4; ++part) issue_part(kt, part);
+    for (int q = 0; q < LPT; ++q) issue_one(kt, q);
   };
 
   // fragment reads: lane reads row lane%32, logical chunk 2*slab + lane/32, into buffer slab&1
@@ -488,12 +482,11 @@ __global__ __launch_bounds__(kGemmThreads, 1) void gemm_nt_dma_kernel(const Gemm
   for (int sl = 0; sl < S; ++sl) off_slab[sl] = rl * kRow + swizzle<BK>(rl, 2 * sl + (lane >> 5)) * 16;
   const int a_frag = (wm * TM * 32) * kRow, b_frag = BM * kRow + (wn * TN * 32) * kRow;
   u32x4_t af[2][TM], bf[2][TN];
-  auto read_frags = [&](int kt, int slab) {
+  // fragment f of a slab: 0 .. TM-1 activation rows, TM .. TM+TN-1 weight rows
+  auto read_one = [&](int kt, int slab, int f) __attribute__((always_inline)) {
     const uint8_t* st = lds + (kt % NS) * kStageBytes + off_slab[slab];
-#pragma unroll
-    for (int i = 0; i < TM; ++i) af[slab & 1][i] = *(const u32x4_t*)(st + a_frag + i * 32 * kRow);
-#pragma unroll
-    for (int j = 0; j < TN; ++j) bf[slab & 1][j] = *(const u32x4_t*)(st + b_frag + j * 32 * kRow);
+    if (f < TM) af[slab & 1][f] = *(const u32x4_t*)(st + a_frag + f * 32 * kRow);
+    else bf[slab & 1][f - TM] = *(const u32x4_t*)(st + b_frag + (f - TM) * 32 * kRow);
   };
 
   f32x16_t acc[TM][TN];
@@ -503,29 +496,49 @@ __global__ __launch_bounds__(kGemmThreads, 1) void gemm_nt_dma_kernel(const Gemm
     for (int j = 0; j < TN; ++j)
 #pragma unroll
       for (int q = 0; q < 16; ++q) acc[i][j][q] = 0.f;
-  // half of a slab's MFMAs (tiles with linear index in [h, h+1) * TM*TN/2), operands in buffer b
-  auto mfma_half = [&](int b, int h) {
+
+  // One slab = TM*TN MFMAs.  Every MFMA keeps the matrix pipeline busy for 32 cycles, during which
+  // this wave may issue other instructions for free -- but a burst of memory instructions takes longer
+  // to issue than that and stalls the MFMAs behind it (8 ds_read_b128 in a row cost 9 % of a 16-MFMA
+  // slab, one behind each MFMA costs 1 %).  So the memory work of a slab is dealt out behind its MFMAs,
+  // a slot each: first the TM + TN fragment reads of the FOLLOWING slab (into the other fragment
+  // buffer), then, where a tile is to be fetched, half of that tile's LDS-DMA loads (a tile's loads are
+  // issued over two slabs).  The compiler waits for all outstanding LDS reads in front of the next
+  // slab's first MFMA; the last read was issued at least TM*TN - (TM+TN) MFMAs earlier.
+  constexpr int kMf = TM * TN, kReads = TM + TN, kDmaPerSlab = LPT / 2;
+  static_assert(LPT % 2 == 0, "a tile's loads are issued in two halves");
+  // kFetch: this slab has slots for loads; they are issued when fetch_kt >= 0 (a scalar branch around
+  // each load: control flow around the MFMAs themselves would make the accumulators phi nodes).
+  auto slab_step = [&](auto fetch_tag, auto sl_tag, auto next_slab_tag, int next_kt, int fetch_kt, int half) __attribute__((always_inline)) {
+    constexpr bool kFetch = decltype(fetch_tag)::value;
+    constexpr int sl = decltype(sl_tag)::value, next_slab = decltype(next_slab_tag)::value;
+    constexpr int kOps = kReads + (kFetch ? kDmaPerSlab : 0);
+    constexpr int kPerSlot = (kOps + kMf - 1) / kMf;
 #pragma unroll
-    for (int ij = 0; ij < TM * TN; ++ij) {
-      if ((ij * 2) / (TM * TN) != h) continue;
+    for (int ij = 0; ij < kMf; ++ij) {
       const int i = ij / TN, j = ij % TN;
-      acc[i][j] = mfma32<DT>(bf[b][j], af[b][i], acc[i][j]);
+      acc[i][j] = mfma32<DT>(bf[sl & 1][j], af[sl & 1][i], acc[i][j]);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int u = 0; u < kPerSlot; ++u) {
+        const int op = ij * kPerSlot + u;
+        if (op < kReads) read_one(next_kt, next_slab, op);
+        else if (kFetch && op < kOps) { if (fetch_kt >= 0) issue_one(fetch_kt, half * kDmaPerSlab + (op - kReads)); }
+      }
+      __builtin_amdgcn_sched_barrier(0);
     }
   };
-  // slab `sl` of a tile while the fragments of the following slab are fetched.  The reads are
-  // issued in the MIDDLE of the slab's MFMAs: the wait the compiler places in front of every
-  // MFMA group covers all LDS reads, so they must be old by the time the next group starts.
-  // `fetch_kt` >= 0: also issue parts `part0` and `part0+1` of that tile's loads, one per MFMA group.
-  auto slab_then_read = [&](int sl, int next_kt, int next_slab, int fetch_kt = -1, int part0 = 0) {
-    mfma_half(sl & 1, 0);
-    __builtin_amdgcn_sched_barrier(0);
-    read_frags(next_kt, next_slab);
-    if (fetch_kt >= 0) issue_part(fetch_kt, part0);
-    __builtin_amdgcn_sched_barrier(0);
-    mfma_half(sl & 1, 1);
-    __builtin_amdgcn_sched_barrier(0);
-    if (fetch_kt >= 0) issue_part(fetch_kt, part0 + 1);
-    __builtin_amdgcn_sched_barrier(0);
+  auto slab_then_read = [&](auto sl_tag, auto next_slab_tag, int next_kt) __attribute__((always_inline)) {
+    slab_step(std::false_type{}, sl_tag, next_slab_tag, next_kt, -1, 0);
+  };
+  auto slab_then_read_fetch = [&](auto sl_tag, auto next_slab_tag, int next_kt, int fetch_kt, int half) __attribute__((always_inline)) {
+    slab_step(std::true_type{}, sl_tag, next_slab_tag, next_kt, fetch_kt, half);
+  };
+  // slabs 1 .. S-2 of a tile (no loads are issued during them)
+  auto middle_slabs = [&](int kt) __attribute__((always_inline)) {
+    if constexpr (S >= 3) slab_then_read(std::integral_constant<int, 1>{}, std::integral_constant<int, 2>{}, kt);
+    if constexpr (S >= 4) slab_then_read(std::integral_constant<int, 2>{}, std::integral_constant<int, 3>{}, kt);
+    static_assert(S <= 4, "at most four slabs per tile");
   };
 
   const int num_kt = g.K / BK;
@@ -542,32 +555,25 @@ __global__ __launch_bounds__(kGemmThreads, 1) void gemm_nt_dma_kernel(const Gemm
   wait_tile(min(NS, num_kt) - 1 < NS - 2 ? min(NS, num_kt) - 1 : NS - 2);
   __builtin_amdgcn_s_barrier();
   OMNI_STAMP(1);
-  read_frags(0, 0);
-  int fetch = -1;                             // tile whose loads are half issued (parts 0,1 done)
-  for (int kt = 0; kt < num_kt - 1; ++kt) {
-    slab_then_read(0, kt, 1, fetch, 2);       // S >= 2: slab 0 is never the tile's last
 #pragma unroll
-    for (int sl = 1; sl < S - 1; ++sl) slab_then_read(sl, kt, sl + 1);
+  for (int f = 0; f < kReads; ++f) read_one(0, 0, f);
+  int fetch = -1;                             // tile whose loads are half issued
+  for (int kt = 0; kt < num_kt - 1; ++kt) {
+    slab_then_read_fetch(std::integral_constant<int, 0>{}, std::integral_constant<int, 1>{}, kt, fetch, 1);   // S >= 2: slab 0 is never the tile's last
+    middle_slabs(kt);
     wait_lds_reads();                         // this wave holds every fragment of tile kt
     // tiles kt+1 .. min(kt+NS-1, num_kt-1) are outstanding; tile kt+1 must have landed
     const int younger = num_kt - 2 - kt;
-#ifndef OMNI_DBG_NO_DMA
     wait_tile(younger < NS - 2 ? younger : NS - 2);
-#endif
-#ifndef OMNI_DBG_NO_BARRIER
     __builtin_amdgcn_s_barrier();             // tile kt+1 visible to all; stage of tile kt free
-#endif
     fetch = (kt + NS < num_kt) ? kt + NS : -1;
-#ifdef OMNI_DBG_NO_DMA
-    fetch = -1;
-#endif
     __builtin_amdgcn_sched_barrier(0);
-    slab_then_read(S - 1, kt + 1, 0, fetch, 0);
+    slab_then_read_fetch(std::integral_constant<int, S - 1>{}, std::integral_constant<int, 0>{}, kt + 1, fetch, 0);
   }
+  slab_then_read(std::integral_constant<int, 0>{}, std::integral_constant<int, 1>{}, num_kt - 1);   // last tile
+  middle_slabs(num_kt - 1);
 #pragma unroll
-  for (int sl = 0; sl < S - 1; ++sl) slab_then_read(sl, num_kt - 1, sl + 1);   // last tile
-  mfma_half((S - 1) & 1, 0);
-  mfma_half((S - 1) & 1, 1);
+  for (int ij = 0; ij < kMf; ++ij) acc[ij / TN][ij % TN] = mfma32<DT>(bf[(S - 1) & 1][ij % TN], af[(S - 1) & 1][ij / TN], acc[ij / TN][ij % TN]);
   OMNI_STAMP(2);
   gemm_epilogue<DT, TM, TN, EPI>(g, acc, m0, n0, wm, wn, lane);
   OMNI_STAMP(3);

@@ -65,19 +65,21 @@ extern "C" OMNI_API int32_t omni_moe_fwd(const void* x, const void* gate_weight,
     if ((he = hipEventRecord((hipEvent_t)fork_event, main_s)) != hipSuccess) return OMNI_ERR_HIP_BASE + (int)he;
     if ((he = hipStreamWaitEvent(branch, (hipEvent_t)fork_event, 0)) != hipSuccess) return OMNI_ERR_HIP_BASE + (int)he;
   }
-  int e;
-  if ((e = omni_router_fwd(x, router_weight_x, router_weight_y, running_mean_x, running_var_x, num_batches_tracked_x,
-                           running_mean_y, running_var_y, num_batches_tracked_y, training, momentum, eps, gates, ids, nullptr,
-                           num_tokens, hidden_size, num_expert_sqrt, num_experts_per_token, dtype, stats_dtype, router_ws, branch)))
+  // From here on the side stream may hold work: whatever happens, the caller's stream is made to wait
+  // for it before this call returns, so that an error leaves no work behind that the caller cannot order.
+  int e = omni_router_fwd(x, router_weight_x, router_weight_y, running_mean_x, running_var_x, num_batches_tracked_x,
+                          running_mean_y, running_var_y, num_batches_tracked_y, training, momentum, eps, gates, ids, nullptr,
+                          num_tokens, hidden_size, num_expert_sqrt, num_experts_per_token, dtype, stats_dtype, router_ws, branch);
+  if (!e) e = omni_swiglu_linear_fwd(x, gate_weight, up_weight, h, num_tokens, hidden_size, intermediate_size, dtype, main_s);
+  if (!e) e = omni_expert_fwd(x, up_embed, down_embed, gates, ids, experts, num_tokens, hidden_size, num_experts,
+                              num_experts_per_token, dtype, OMNI_EXPERT_ALGO_AUTO, expert_ws, branch);
+  if (!side_stream) {   // one stream: the add is the down projection's epilogue
+    if (!e) e = omni_linear_fwd(h, down_weight, experts, y, num_tokens, intermediate_size, hidden_size, dtype, main_s);
     return e;
-  if ((e = omni_swiglu_linear_fwd(x, gate_weight, up_weight, h, num_tokens, hidden_size, intermediate_size, dtype, main_s))) return e;
-  if ((e = omni_expert_fwd(x, up_embed, down_embed, gates, ids, experts, num_tokens, hidden_size, num_experts,
-                           num_experts_per_token, dtype, OMNI_EXPERT_ALGO_AUTO, expert_ws, branch)))
-    return e;
-  if (!side_stream)   // one stream: the add is the down projection's epilogue
-    return omni_linear_fwd(h, down_weight, experts, y, num_tokens, intermediate_size, hidden_size, dtype, main_s);
-  if ((e = omni_linear_fwd(h, down_weight, nullptr, y, num_tokens, intermediate_size, hidden_size, dtype, main_s))) return e;
-  if ((he = hipEventRecord((hipEvent_t)join_event, branch)) != hipSuccess) return OMNI_ERR_HIP_BASE + (int)he;
-  if ((he = hipStreamWaitEvent(main_s, (hipEvent_t)join_event, 0)) != hipSuccess) return OMNI_ERR_HIP_BASE + (int)he;
+  }
+  if (!e) e = omni_linear_fwd(h, down_weight, nullptr, y, num_tokens, intermediate_size, hidden_size, dtype, main_s);
+  if ((he = hipEventRecord((hipEvent_t)join_event, branch)) != hipSuccess) return e ? e : OMNI_ERR_HIP_BASE + (int)he;
+  if ((he = hipStreamWaitEvent(main_s, (hipEvent_t)join_event, 0)) != hipSuccess) return e ? e : OMNI_ERR_HIP_BASE + (int)he;
+  if (e) return e;
   return omni_add_inplace(y, experts, (int64_t)T * hidden_size, dtype, main_s);
 }
