@@ -152,6 +152,13 @@ OMNI_API int32_t omni_swiglu_linear_fwd(const void* x, const void* gate_weight, 
 OMNI_API int32_t omni_linear_fwd(const void* x, const void* weight, const void* residual, void* y, int64_t num_tokens,
                                  int32_t in_features, int32_t out_features, int32_t dtype, void* stream);
 
+/* Diagnostic, no counterpart in the reference: the device's matrix-core rate with nothing else going on.
+ * num_blocks blocks of 4 waves each issue iters x 16 v_mfma_f32_32x32x16_bf16 (iters * 16 * 32768 flop per
+ * wave) on register operands read once from `operands` (8 KiB; the bits matter: the clock the board sustains
+ * under its power limit depends on how many of them toggle).  sink: num_blocks * 256 floats, overwritten.
+ * The caller times the launch; the benchmark prints the result beside the published peak. */
+OMNI_API int32_t omni_probe_mfma(const void* operands, float* sink, int32_t num_blocks, int32_t iters, void* stream);
+
 /* y[i] = round(y[i] + addend[i]) in place: the layer's final  mlp + experts  (omni_moe.py:102) as a
  * call of its own, for callers that run the two branches on different streams.  num_elements a
  * multiple of 8 (4 for f32); both pointers 16-byte aligned. */

@@ -796,3 +796,39 @@ extern "C" OMNI_API int32_t omni_add_inplace(void* y, const void* addend, int64_
   else hipLaunchKernelGGL(add_inplace_kernel<kF32>, dim3(blocks), dim3(256), 0, s, (uint8_t*)y, (const uint8_t*)addend, chunks);
   return omni::to_code(hipGetLastError());
 }
+
+namespace omni {
+// Matrix-core rate with nothing else going on: every wave keeps 16 accumulator tiles and issues
+// MFMAs on operands it read once (8 KiB of caller data, so that the operand bits are realistic:
+// the sustained clock under the board's power limit depends on how many bits toggle).
+__global__ __launch_bounds__(kGemmThreads, 1) void mfma_probe_kernel(const u32x4_t* __restrict__ operands, float* __restrict__ sink, int iters) {
+  f32x16_t acc[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i)
+#pragma unroll
+    for (int q = 0; q < 16; ++q) acc[i][q] = 0.f;
+  u32x4_t a[4], b[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    a[i] = operands[(threadIdx.x * 8 + i) & 511];
+    b[i] = operands[(threadIdx.x * 8 + 4 + i) & 511];
+  }
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[i] = mfma32<kBF16>(a[i & 3], b[i >> 2], acc[i]);
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) s += acc[i][0] + acc[i][5];
+  sink[blockIdx.x * kGemmThreads + threadIdx.x] = s;
+}
+}  // namespace omni
+
+extern "C" OMNI_API int32_t omni_probe_mfma(const void* operands, float* sink, int32_t num_blocks, int32_t iters, void* stream) {
+  if (num_blocks <= 0 || iters <= 0) return OMNI_ERR_SHAPE;
+  if (!operands || !sink) return OMNI_ERR_NULL;
+  hipLaunchKernelGGL(omni::mfma_probe_kernel, dim3(num_blocks), dim3(omni::kGemmThreads), 0, (hipStream_t)stream,
+                     (const omni::u32x4_t*)operands, sink, iters);
+  return omni::to_code(hipGetLastError());
+}
+
