@@ -174,6 +174,9 @@ def test_layer_matches_oracle(case, training, device):
     # tokens whose expert set matches the oracle's must match in value; the others differ by
     # which near-tied expert was picked, which changes y by at most a few gate*|V| -- still small
     torch.testing.assert_close(got.cpu().float(), want.float(), rtol=2e-2, atol=2e-2)
+    # the same bound on the scale of the output (|y| is a few 0.01 at these weights, where a flat 2e-2 says little)
+    scale = want.float().abs().max().item()
+    assert (got.cpu().float() - want.float()).abs().max().item() <= 2e-2 * scale, scale
     if training:
         assert layer.router_norm_x.num_batches_tracked.item() == 1
         torch.testing.assert_close(layer.router_norm_x.running_mean.float().cpu(), bx.running_mean, rtol=2e-2, atol=2e-3)
@@ -268,6 +271,51 @@ def test_layer_config5_large_skewed(device):
     assert set_agree >= 0.999
     torch.testing.assert_close(y.view(-1, H)[sub.to(device)].float().cpu(), want.view(-1, H).float(), rtol=2e-2, atol=2e-2)
     torch.testing.assert_close(gates.cpu()[sub].float(), want_g.float(), rtol=2e-2, atol=2e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("two_streams", [False, True], ids=["one-stream", "two-streams"])
+def test_layer_expert_term_visible_auto_split(two_streams, dtype, device):
+    """A layer whose expert branch is as large as its MLP branch (weights ~ N(0, 0.1)) and whose shape makes the layer call
+    pick the hidden-split expert algorithm (4096 tokens x 8 = 32768 pairs, tables that overflow one L2): y - mlp must equal
+    the oracle's expert term on the expert term's own scale, on one stream and on two.  A layer that dropped or mis-wired
+    router -> experts (wrong gates or ids buffer, workspace overlap, missing join) fails here."""
+    from omni_moe.modules.omni_moe import OmniMoE, OmniMoEConfig
+    T, H, I, N, k = 4096, 512, 512, (1024 if dtype == torch.float32 else 4096), 8
+    x, w = oracle.make_layer_inputs(21, T, H, I, N, dtype=dtype, w_std=0.1)
+    w.down_proj = (w.down_proj.float() * 0.03).to(dtype)     # the shared MLP scaled down to the size of the expert term
+    r = w.router_gate_x.size(0)
+    layer = OmniMoE(OmniMoEConfig(H, I, "silu", N, k))
+    layer.load_state_dict({"gate_proj.weight": w.gate_proj, "up_proj.weight": w.up_proj, "down_proj.weight": w.down_proj,
+                           "router_gate_x.weight": w.router_gate_x, "router_gate_y.weight": w.router_gate_y,
+                           "up_embed.weight": w.up_embed, "down_embed.weight": w.down_embed}, strict=False)
+    layer = layer.to(device=device, dtype=dtype).eval()      # eval: token-independent, the oracle needs no batch statistics
+    layer.overlap_branches = two_streams
+    layer.overlap_min_work = 0
+    from omni_moe.ops.hip import _lib
+    lib = _lib.load()
+    es = 4 if dtype == torch.float32 else 2
+    assert lib.omni_expert_workspace_bytes(T, H, N, k, _lib.DTYPE_CODE[dtype], _lib.ALGO_AUTO) == 8 * T * k * 4, "AUTO should pick the split algorithm here"
+    print(f"layer with visible expert term, {dtype}, two_streams={two_streams}", flush=True)
+    xd = x.to(device)
+    y = layer(xd).view(-1, H)
+    mlp = _ops().hip_omni_mlp_func(xd.view(-1, H), layer.gate_proj.weight, layer.up_proj.weight, layer.down_proj.weight)
+    gates, ids = layer.route(xd.view(-1, H))
+    torch.cuda.synchronize()
+    bx, by = oracle.BNState.fresh(r), oracle.BNState.fresh(r)
+    want_y, want_g, want_i = oracle.moe_forward(x, w, bx, by, k, training=False)
+    # the oracle's expert term for the ids the device chose (near-tied scores may resolve differently in bf16)
+    want_e = oracle.expert_forward(x.view(-1, H), w.up_embed, w.down_embed, gates.cpu(), ids.cpu()).float()
+    e_scale, m_scale = want_e.abs().max().item(), mlp.float().abs().max().item()
+    print(f"   max |experts| {e_scale:.3f}, max |mlp| {m_scale:.3f}")
+    assert e_scale > 0.2 * m_scale                             # the expert term is visible
+    got_e = (y.float() - mlp.float()).cpu()
+    tol = 1e-4 if dtype == torch.float32 else 2e-2            # bf16: y and mlp are rounded to bf16 on the scale of their sum
+    assert (got_e - want_e).abs().max().item() <= tol * (e_scale + m_scale), (got_e - want_e).abs().max().item()
+    assert (got_e - want_e).abs().mean().item() <= 0.1 * tol * (e_scale + m_scale)
+    same = (ids.cpu().sort(-1).values == want_i.sort(-1).values).all(-1)
+    assert same.float().mean().item() >= (0.999 if dtype == torch.float32 else 0.97)
+    torch.testing.assert_close(y.cpu().float()[same], want_y.view(-1, H).float()[same], rtol=tol, atol=tol * (e_scale + m_scale))
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=["bf16", "f32"])

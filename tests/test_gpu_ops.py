@@ -181,6 +181,29 @@ def test_expert_segment_algorithm_equals_gather(case, device):
     assert torch.equal(a, b)
 
 
+@pytest.fixture(scope="module")
+def config3_inputs():
+    """benchmark config 3 at full size, exactly what bench.py times: 16384 tokens, hidden 1024, 4096 experts, k=16, bf16, seed 2;
+    the oracle's output for all 16384 tokens (token chunks of 2048, fp32 sums, one rounding)."""
+    T, H, N, k = 16384, 1024, 4096, 16
+    x, up, down, gates, ids = oracle.make_expert_inputs(2, T, H, N, k)
+    return (x, up, down, gates, ids), oracle.expert_forward(x, up, down, gates, ids)
+
+
+@pytest.mark.parametrize("algo", ["auto", "split", "gather", "segment"])
+def test_expert_config3_full_size(algo, config3_inputs, device):
+    (x, up, down, gates, ids), want = config3_inputs
+    print(f"expert config 3 full size, algo={algo}", flush=True)
+    got = _ops().hip_omni_expert_func(*(t.to(device) for t in (x, up, down, gates, ids)), algo=algo)
+    torch.cuda.synchronize()
+    g, w = got.cpu().float(), want.float()
+    torch.testing.assert_close(g, w, rtol=2e-2, atol=2e-2)
+    # both sum in fp32 and round once: at most one bf16 ulp apart, on the scale of the output (max |y| ~ 0.02)
+    scale = w.abs().max().item()
+    assert (g - w).abs().max().item() <= 1e-2 * scale, ((g - w).abs().max().item(), scale)
+    assert (g != w).float().mean().item() < 0.05          # and most elements are bit-identical
+
+
 def _split_covers(H, dtype):
     slice_bytes = H * torch.empty((), dtype=dtype).element_size() // 8
     return H * torch.empty((), dtype=dtype).element_size() % 128 == 0 and slice_bytes in (64, 128, 256, 512, 1024)
