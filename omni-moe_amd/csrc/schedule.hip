@@ -4,42 +4,51 @@
 // which runs ~12 torch launches including a radix sort and reads two results back to
 // the host (:82, :90).  Here the pairs are sorted by expert id with one counting pass when
 // N <= 4096 (one bin per expert), two passes (low then high half of the id bits) above that.
-// A pass is: per-block bin counts in LDS -> exclusive scan over [bin][block] -> scatter.  The
-// scatter is order preserving without any global atomic: a block owns a contiguous tile of
-// the input, each of its 4 waves a contiguous quarter; per-wave bin bases come from an LDS
-// table, and inside a wave 64 consecutive items rank themselves with ballots.  So a segment
-// lists its pairs by ascending pair id, and the result is bit-identical from run to run.
-// Offsets are dense over all N experts (an unused expert has an empty segment), so no
-// compaction pass is needed, and nothing returns to the host.
+// A pass is two kernels:
+//   count:   every block counts the bins of its contiguous tile of the input in LDS and writes
+//            them as one row of hist[block][bin] (coalesced, 16-bit counters: a tile has fewer
+//            than 65536 pairs; the histogram is the only scratch);
+//   scatter: every block sums the rows of hist (all of them for the bins' totals, the rows above
+//            its own for its share), scans the totals over the bins, and has its output bases;
+//            block 0 writes them out as the segment offsets.  Then it places its tile.
+// The scatter is order preserving without any global atomic: each of the block's 8 waves owns a
+// contiguous eighth of the tile; per-wave bin bases come from an LDS table, and inside a wave 64
+// consecutive items rank themselves with ballots.  So a segment lists its pairs by ascending pair
+// id, and the result is bit-identical from run to run.  Offsets are dense over all N experts (an
+// unused expert has an empty segment), so no compaction pass is needed, and nothing returns to
+// the host.  Few, large tiles (about 131072 / bins blocks) keep the histogram small: it is read
+// once per block.
 #include "common.h"
 #include "omni_moe_hip.h"
 
 namespace omni {
 
-constexpr int kScanBlock = 256;
-constexpr int kScanPerThread = 16;
-constexpr int kScanTile = kScanBlock * kScanPerThread;   // 4096 entries per block
-constexpr int kMaxScanBlocks = 1024;                      // <= 4 Mi entries per scan
-
-constexpr int kSortThreads = 256;
+constexpr int kSortThreads = 512;
 constexpr int kSortWaves = kSortThreads / kWave;
 constexpr int kMaxBins = 4097;                            // 4096 experts (or id slices) + 1 bin for ids outside [0, N)
+constexpr int kBinChunk = 8;                              // bins a thread sums at a time (one 16-byte load per histogram row)
+constexpr int kMaxStride = (kMaxBins + kBinChunk - 1) / kBinChunk * kBinChunk;
+constexpr int kMaxSortBlocks = 1024;
+constexpr int kMaxTile = 63 * 1024;                       // counters are 16 bits wide
+constexpr int kRowBatch = 16;                             // histogram rows whose loads are in flight together
+static_assert(kMaxBins <= kSortThreads * kBinChunk + 1, "the scan covers 8 bins per thread plus one");
 
 struct SortPass {
   const int32_t* keys_in;   // expert ids, in the order left by the previous pass
   const int32_t* vals_in;   // pair ids travelling with them; NULL = position (first pass)
-  int32_t* keys_out;
+  int32_t* keys_out;        // NULL: not needed (single pass)
   int32_t* vals_out;
   int32_t* tok_out;         // NULL, or pair id / top_k (last pass)
-  int32_t* hist;            // [bins][blocks]: counts, then (after the scan) output bases
+  int32_t* offsets_out;     // NULL, or [bins]: first output position of every bin (single pass: the segment offsets)
+  uint16_t* hist;           // [blocks][stride] bin counts of every tile
   int64_t num_pairs;
-  int tile;                 // pairs per block, a multiple of 256
-  int blocks, bins, bits;   // bits = ceil(log2(bins))
+  int tile;                 // pairs per block, a multiple of 1024
+  int blocks, bins, stride, bits;   // stride = bins rounded up to 8; bits = ceil(log2(bins))
   int shift;                // digit = id >> shift ...
   uint32_t mask;            //   ... & mask (0xFFFFFFFF on the last pass)
   int last;                 // last pass: ids outside [0, N) go to bin bins-1; earlier passes: to bin 0
   uint32_t num_experts;
-  int top_k;
+  uint64_t inv_top_k;       // ceil(2^40 / top_k): (v * inv_top_k) >> 40 == v / top_k for every v < 2^31 and top_k <= 2^9
 };
 
 __device__ __forceinline__ int sort_digit(const SortPass& a, int32_t key) {
@@ -50,50 +59,118 @@ __device__ __forceinline__ int sort_digit(const SortPass& a, int32_t key) {
 
 __global__ __launch_bounds__(kSortThreads) void sort_count_kernel(const SortPass a) {
   extern __shared__ int32_t cnt[];
-  for (int d = threadIdx.x; d < a.bins; d += kSortThreads) cnt[d] = 0;
+  for (int d = threadIdx.x; d < a.stride; d += kSortThreads) cnt[d] = 0;
   __syncthreads();
   const int64_t t0 = (int64_t)blockIdx.x * a.tile;
   const int64_t t1 = t0 + a.tile < a.num_pairs ? t0 + a.tile : a.num_pairs;
   for (int64_t i = t0 + threadIdx.x; i < t1; i += kSortThreads) atomicAdd(&cnt[sort_digit(a, a.keys_in[i])], 1);
   __syncthreads();
-  for (int d = threadIdx.x; d < a.bins; d += kSortThreads) a.hist[(int64_t)d * a.blocks + blockIdx.x] = cnt[d];
+  for (int d = threadIdx.x; d < a.stride; d += kSortThreads) a.hist[(int64_t)blockIdx.x * a.stride + d] = (uint16_t)cnt[d];
 }
 
 __global__ __launch_bounds__(kSortThreads) void sort_scatter_kernel(const SortPass a) {
-  extern __shared__ int32_t tbl[];                       // [waves][bins]: counts, then running output positions
+  extern __shared__ int32_t tbl[];                       // [waves][stride]: counts, then running output positions; then [stride] bin bases
+  __shared__ int32_t wave_tot[kSortWaves];
+  int32_t* bin_base = tbl + kSortWaves * a.stride;
   const int lane = lane_id(), wave = threadIdx.x >> 6;
-  for (int d = threadIdx.x; d < a.bins * kSortWaves; d += kSortThreads) tbl[d] = 0;
+  for (int d = threadIdx.x * 4; d < a.stride * kSortWaves; d += kSortThreads * 4) *(u32x4_t*)(tbl + d) = u32x4_t{0, 0, 0, 0};   // stride % 8 == 0
   __syncthreads();
   const int64_t t0 = (int64_t)blockIdx.x * a.tile;
   const int64_t t1 = t0 + a.tile < a.num_pairs ? t0 + a.tile : a.num_pairs;
-  const int64_t w0 = t0 + (int64_t)wave * (a.tile / kSortWaves);                  // this wave's quarter, in order
-  const int64_t w1 = w0 + a.tile / kSortWaves < t1 ? w0 + a.tile / kSortWaves : t1;
-  int32_t* mine = tbl + wave * a.bins;
+  const int per_wave = a.tile / kSortWaves;
+  const int64_t w0 = t0 + (int64_t)wave * per_wave < t1 ? t0 + (int64_t)wave * per_wave : t1;   // this wave's eighth, in order
+  const int64_t w1 = w0 + per_wave < t1 ? w0 + per_wave : t1;
+  int32_t* mine = tbl + wave * a.stride;
   for (int64_t i = w0 + lane; i < w1; i += kWave) atomicAdd(&mine[sort_digit(a, a.keys_in[i])], 1);
   __syncthreads();
-  // bases: the block's base of a bin, then wave by wave.  The strided global reads of a thread's
-  // bins are all issued before any is used.
-  constexpr int kBinsPerThread = (kMaxBins + kSortThreads - 1) / kSortThreads;
-  int32_t block_base[kBinsPerThread];
+
+  // Output bases.  Thread t takes bins 8t .. 8t+7 and walks down the histogram rows: the rows above this block's
+  // give what earlier tiles put into each bin, all rows the bin's total.  An exclusive scan of the totals over the
+  // bins (thread order = bin order) gives each bin's first position.  The rows come from other blocks' writes, i.e.
+  // from memory: the loads of kRowBatch rows are in flight together.  512 threads cover 4096 bins; the one bin
+  // beyond them (ids outside the table, when there are 4096 experts) is summed by wave 0, a row per lane.
+  const int d0 = threadIdx.x * kBinChunk;
+  const bool active = d0 < a.stride && d0 < kSortThreads * kBinChunk;
+  int32_t before[kBinChunk], rest[kBinChunk];
 #pragma unroll
-  for (int j = 0; j < kBinsPerThread; ++j) {
-    const int d = threadIdx.x + j * kSortThreads;
-    block_base[j] = d < a.bins ? a.hist[(int64_t)d * a.blocks + blockIdx.x] : 0;
+  for (int i = 0; i < kBinChunk; ++i) before[i] = rest[i] = 0;
+  auto add_rows = [&](int32_t (&acc)[kBinChunk], int first, int end) {
+    for (int b0 = first; b0 < end; b0 += kRowBatch) {
+      u32x4_t row[kRowBatch];
+#pragma unroll
+      for (int j = 0; j < kRowBatch; ++j)
+        row[j] = (active && b0 + j < end) ? *(const u32x4_t*)(a.hist + (int64_t)(b0 + j) * a.stride + d0) : u32x4_t{0, 0, 0, 0};
+#pragma unroll
+      for (int j = 0; j < kRowBatch; ++j)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const uint32_t pair = row[j][i];
+          acc[2 * i] += (int32_t)(pair & 0xffffu);
+          acc[2 * i + 1] += (int32_t)(pair >> 16);
+        }
+    }
+  };
+  add_rows(before, 0, (int)blockIdx.x);
+  add_rows(rest, (int)blockIdx.x, a.blocks);
+  const int tail_bin = kSortThreads * kBinChunk;         // 4096
+  int32_t tail_before = 0, tail_total = 0;
+  if (a.bins > tail_bin && wave == 0) {
+    for (int b = lane; b < a.blocks; b += kWave) {
+      const int32_t c = a.hist[(int64_t)b * a.stride + tail_bin];
+      tail_total += c;
+      tail_before += b < (int)blockIdx.x ? c : 0;
+    }
+#pragma unroll
+    for (int m = kWave / 2; m >= 1; m >>= 1) {
+      tail_total += __shfl_xor(tail_total, m, kWave);
+      tail_before += __shfl_xor(tail_before, m, kWave);
+    }
   }
+  {
+    int32_t tsum = 0;
 #pragma unroll
-  for (int j = 0; j < kBinsPerThread; ++j) {
-    const int d = threadIdx.x + j * kSortThreads;
-    if (d < a.bins) {
-      int32_t base = block_base[j];
+    for (int i = 0; i < kBinChunk; ++i) tsum += before[i] + rest[i];
+    int32_t inc = tsum;                                  // inclusive scan across the wave
 #pragma unroll
-      for (int w = 0; w < kSortWaves; ++w) {
-        const int32_t c = tbl[w * a.bins + d];
-        tbl[w * a.bins + d] = base;
-        base += c;
+    for (int d = 1; d < kWave; d <<= 1) {
+      const int32_t o = __shfl_up(inc, d, kWave);
+      if (lane >= d) inc += o;
+    }
+    if (lane == kWave - 1) wave_tot[wave] = inc;
+    __syncthreads();
+    int32_t excl = inc - tsum, all = 0;
+#pragma unroll
+    for (int w = 0; w < kSortWaves; ++w) {
+      excl += w < wave ? wave_tot[w] : 0;
+      all += wave_tot[w];
+    }
+#pragma unroll
+    for (int i = 0; i < kBinChunk; ++i) {
+      const int d = d0 + i;
+      if (active && d < a.bins) {
+        if (a.offsets_out && blockIdx.x == 0) a.offsets_out[d] = excl;
+        bin_base[d] = excl + before[i];
       }
+      excl += before[i] + rest[i];
+    }
+    if (a.bins > tail_bin && threadIdx.x == 0) {         // the bin behind all others starts where they end
+      if (a.offsets_out && blockIdx.x == 0) a.offsets_out[tail_bin] = all;
+      bin_base[tail_bin] = all + tail_before;
+    }
+    __syncthreads();
+  }
+  // per-wave bases: consecutive threads take consecutive bins (no bank conflicts), wave by wave down the table
+  for (int d = threadIdx.x; d < a.bins; d += kSortThreads) {
+    int32_t base = bin_base[d];
+#pragma unroll
+    for (int w = 0; w < kSortWaves; ++w) {
+      const int32_t c = tbl[w * a.stride + d];
+      tbl[w * a.stride + d] = base;
+      base += c;
     }
   }
   __syncthreads();
+
   const uint64_t below = (1ull << lane) - 1ull;
   constexpr int kGroup = 8;                                  // steps whose loads are issued together
   for (int64_t g0 = w0; g0 < w1; g0 += kGroup * kWave) {
@@ -110,25 +187,33 @@ __global__ __launch_bounds__(kSortThreads) void sort_scatter_kernel(const SortPa
       const bool active = i < w1;
       const int32_t key = keys[u], val = vals[u];
       const int d = active ? sort_digit(a, key) : 0;
-      uint64_t same = __ballot(active);                      // lanes holding the same bin as this one
-      for (int b = 0; b < a.bits; ++b) {
-        const bool bit = (d >> b) & 1;
-        const uint64_t vote = __ballot(bit && active);
-        same &= bit ? vote : ~vote;
-      }
-      const int rank = __popcll(same & below);
+      // Position = the bin's running base + the number of earlier lanes of this step with the same bin.  Every lane
+      // reads the base, then bumps it; a lane that finds the base already bumped shares its bin with another lane of
+      // the step.  Only then are the lanes of that bin ranked by lane number (whatever order the adds took effect in).
+      int32_t pos = 0, bumped = 0;
       if (active) {
-        const int32_t pos = mine[d] + rank;
-        a.keys_out[pos] = key;
+        pos = mine[d];
+        bumped = atomicAdd(&mine[d], 1);
+      }
+      uint64_t shared = __ballot(active && bumped != pos);   // the non-first lanes of shared bins
+      while (shared) {
+        const int l = __builtin_ctzll(shared);
+        const int v = __shfl(d, l, kWave);
+        const uint64_t grp = __ballot(active && d == v);     // all lanes of that bin; they read the same base
+        if (active && d == v) pos += __popcll(grp & below);
+        shared &= ~grp;
+      }
+      if (active) {
+        if (a.keys_out) a.keys_out[pos] = key;
         a.vals_out[pos] = val;
-        if (a.tok_out) a.tok_out[pos] = val / a.top_k;
-        if (rank == 0) mine[d] += __popcll(same);          // one lane per bin; LDS ops of a wave execute in order
+        if (a.tok_out) a.tok_out[pos] = (int32_t)(((uint64_t)(uint32_t)val * a.inv_top_k) >> 40);   // val / top_k
       }
     }
   }
 }
 
-// offsets[e] = first position whose (sorted) id is >= e; ids outside [0, N) count as N.
+// offsets[e] = first position whose (sorted) id is >= e; ids outside [0, N) count as N.  Two-pass sorts only:
+// their last pass has a bin per high half of the id, not per expert.
 __global__ __launch_bounds__(256) void segment_offsets_kernel(const int32_t* __restrict__ sorted_keys, int32_t* __restrict__ offsets,
                                                               int64_t num_pairs, uint32_t num_experts) {
   for (int64_t i = blockIdx.x * 256ll + threadIdx.x; i <= num_pairs; i += gridDim.x * 256ll) {
@@ -140,76 +225,18 @@ __global__ __launch_bounds__(256) void segment_offsets_kernel(const int32_t* __r
   }
 }
 
-// Phase 1: every block scans its tile of 4096 bins locally (exclusive), leaves the
-// tile total in tile_sums[block].
-__global__ __launch_bounds__(kScanBlock) void scan_tiles_kernel(const int32_t* counts, int32_t* offsets,   // may alias: a thread reads its entries before it writes them
-                                                                int32_t* __restrict__ tile_sums, int64_t n) {
-  __shared__ int32_t wave_tot[kScanBlock / kWave];
-  const int64_t base = (int64_t)blockIdx.x * kScanTile + threadIdx.x * kScanPerThread;
-  int32_t v[kScanPerThread], sum = 0;
-#pragma unroll
-  for (int i = 0; i < kScanPerThread; ++i) {
-    v[i] = (base + i < n) ? counts[base + i] : 0;
-    sum += v[i];
-  }
-  // inclusive scan of the per-thread sums across the wave
-  int32_t inc = sum;
-  const int lane = lane_id(), wave = threadIdx.x >> 6;
-#pragma unroll
-  for (int d = 1; d < kWave; d <<= 1) {
-    const int32_t o = __shfl_up(inc, d, kWave);
-    if (lane >= d) inc += o;
-  }
-  if (lane == kWave - 1) wave_tot[wave] = inc;
-  __syncthreads();
-  int32_t before = inc - sum;
-  for (int w = 0; w < wave; ++w) before += wave_tot[w];
-#pragma unroll
-  for (int i = 0; i < kScanPerThread; ++i) {
-    if (base + i < n) offsets[base + i] = before;
-    before += v[i];
-  }
-  if (threadIdx.x == kScanBlock - 1) tile_sums[blockIdx.x] = before;
-}
-
-// Phase 2: add the sum of the preceding tiles; also seed the scatter cursors and
-// write offsets[n] = total.
-__global__ __launch_bounds__(kScanBlock) void scan_fixup_kernel(int32_t* __restrict__ offsets, int32_t* __restrict__ cursor,
-                                                                const int32_t* __restrict__ tile_sums, int64_t n, int num_tiles) {
-  __shared__ int32_t wave_tot[kScanBlock / kWave];
-  int32_t part = 0;
-  for (int i = threadIdx.x; i < (int)blockIdx.x; i += kScanBlock) part += tile_sums[i];
-  int32_t w = part;
-#pragma unroll
-  for (int m = kWave / 2; m >= 1; m >>= 1) w += __shfl_xor(w, m, kWave);
-  if (lane_id() == 0) wave_tot[threadIdx.x >> 6] = w;
-  __syncthreads();
-  int32_t prior = 0;
-#pragma unroll
-  for (int i = 0; i < kScanBlock / kWave; ++i) prior += wave_tot[i];
-  const int64_t base = (int64_t)blockIdx.x * kScanTile + threadIdx.x * kScanPerThread;
-#pragma unroll
-  for (int i = 0; i < kScanPerThread; ++i)
-    if (base + i < n) {
-      const int32_t o = offsets[base + i] + prior;
-      offsets[base + i] = o;
-      if (cursor) cursor[base + i] = o;
-    }
-  if ((int)blockIdx.x == num_tiles - 1 && threadIdx.x == 0) offsets[n] = prior + tile_sums[num_tiles - 1];
-}
-
 static inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 static inline int ceil_log2(uint64_t v) { int b = 0; while ((1ull << b) < v) ++b; return b; }
 
 // How the sort of P pairs with ids below N is split into passes and tiles.
 struct SortPlan {
-  int passes, lo_bits, bins[2], tile, blocks;
+  int passes, lo_bits, bins[2], stride, tile, blocks;
   size_t hist_entries;
 };
 static bool make_plan(int64_t P, int64_t N, SortPlan* pl) {
   const int kb = ceil_log2((uint64_t)N);
-  if (kb <= 12) { pl->passes = 1; pl->lo_bits = 0; pl->bins[0] = (int)N + 1; pl->bins[1] = 0; }
+  if (N + 1 <= kMaxBins) { pl->passes = 1; pl->lo_bits = 0; pl->bins[0] = (int)N + 1; pl->bins[1] = 0; }
   else {
     pl->passes = 2; pl->lo_bits = kb / 2;
     pl->bins[0] = 1 << pl->lo_bits;
@@ -217,25 +244,32 @@ static bool make_plan(int64_t P, int64_t N, SortPlan* pl) {
   }
   const int maxb = pl->bins[0] > pl->bins[1] ? pl->bins[0] : pl->bins[1];
   if (maxb > kMaxBins) return false;                       // N > 16 Mi experts
-  int tile = 2048;
-  while ((int64_t)maxb * ((P + tile - 1) / tile) > (int64_t)kMaxScanBlocks * kScanTile && tile < (1 << 20)) tile *= 2;
-  if ((int64_t)maxb * ((P + tile - 1) / tile) > (int64_t)kMaxScanBlocks * kScanTile) return false;
-  pl->tile = tile;
+  pl->stride = (maxb + kBinChunk - 1) / kBinChunk * kBinChunk;
+  // every block reads the whole histogram: about 128 Ki counters of it (32 tiles at 4097 bins, 256 at 512),
+  // more where a tile would outgrow its 16-bit counters
+  int want = ((1 << 17) + maxb - 1) / maxb;
+  want = want < 1 ? 1 : (want > 256 ? 256 : want);
+  int64_t tile = (P + want - 1) / want;
+  tile = (tile + 1023) / 1024 * 1024;
+  if (tile < 1024) tile = 1024;
+  if (tile > kMaxTile) tile = kMaxTile;
+  if ((P + tile - 1) / tile > kMaxSortBlocks) return false;   // more than 64 Mi pairs
+  pl->tile = (int)tile;
   pl->blocks = (int)((P + tile - 1) / tile);
   if (pl->blocks < 1) pl->blocks = 1;
-  pl->hist_entries = (size_t)maxb * pl->blocks;
+  pl->hist_entries = (size_t)pl->stride * pl->blocks;
   return true;
 }
 
 }  // namespace omni
 
-// workspace: hist [maxbins*blocks + 1] | scan tile sums [1024] | keys A [P] | keys B [P] | pair ids [P]
+// workspace: hist [blocks][stride] | two-pass sorts only: keys A [P] | keys B [P] | pair ids [P]
 extern "C" OMNI_API size_t omni_schedule_workspace_bytes(int64_t num_tokens, int32_t num_experts_per_token, int64_t num_experts) {
   using namespace omni;
   const int64_t P = num_tokens * (int64_t)num_experts_per_token;
   SortPlan pl;
   if (num_tokens < 0 || num_experts_per_token < 0 || num_experts <= 0 || !make_plan(P, num_experts, &pl)) return 0;
-  return align_up((pl.hist_entries + 1) * 4, 256) + align_up((size_t)kMaxScanBlocks * 4, 256) + 3 * align_up((size_t)P * 4 + 4, 256);
+  return align_up(pl.hist_entries * 2, 256) + (pl.passes == 2 ? 3 * align_up((size_t)P * 4 + 4, 256) : 0);
 }
 
 extern "C" OMNI_API int32_t omni_schedule(const int32_t* indices, int32_t* offsets, int32_t* sorted_pair_ids,
@@ -250,47 +284,46 @@ extern "C" OMNI_API int32_t omni_schedule(const int32_t* indices, int32_t* offse
   if (!workspace) return OMNI_ERR_WORKSPACE;
   hipStream_t s = (hipStream_t)stream;
   char* w = (char*)workspace;
-  int32_t* hist = (int32_t*)w;       w += align_up((pl.hist_entries + 1) * 4, 256);
-  int32_t* tile_sums = (int32_t*)w;  w += align_up((size_t)kMaxScanBlocks * 4, 256);
-  int32_t* keys_a = (int32_t*)w;     w += align_up((size_t)P * 4 + 4, 256);
+  uint16_t* hist = (uint16_t*)w;     w += align_up(pl.hist_entries * 2, 256);
+  int32_t* keys_a = (int32_t*)w;     w += align_up((size_t)P * 4 + 4, 256);      // the three arrays exist for two-pass sorts only
   int32_t* keys_b = (int32_t*)w;     w += align_up((size_t)P * 4 + 4, 256);
   int32_t* vals_a = (int32_t*)w;
 
-  const int32_t* sorted_keys = indices;                     // P == 0: nothing to sort
-  if (P > 0) {
+  static std::atomic<uint64_t> configured{0};              // tables of up to 8 x 4104 counters exceed the 64 KiB default
+  if (hipError_t e = ensure_dynamic_lds((const void*)sort_scatter_kernel, kMaxStride * (kSortWaves + 1) * 4, configured); e != hipSuccess)
+    return OMNI_ERR_HIP_BASE + (int)e;
+  const bool single = pl.passes == 1;
+  if (single || P > 0) {
     for (int pass = 0; pass < pl.passes; ++pass) {
       const bool last = pass == pl.passes - 1;
       SortPass a;
       a.keys_in = pass == 0 ? indices : keys_a;
       a.vals_in = pass == 0 ? nullptr : vals_a;
-      a.keys_out = last ? keys_b : keys_a;
+      a.keys_out = single ? nullptr : (last ? keys_b : keys_a);
       a.vals_out = last ? sorted_pair_ids : vals_a;
       a.tok_out = last ? sorted_token_ids : nullptr;
+      a.offsets_out = single ? offsets : nullptr;          // one bin per expert: the bins' first positions ARE the offsets
       a.hist = hist;
       a.num_pairs = P;
       a.tile = pl.tile;
       a.blocks = pl.blocks;
       a.bins = pl.bins[pass];
+      a.stride = pl.stride;
       a.bits = ceil_log2((uint64_t)a.bins);
       a.shift = pass == 0 ? 0 : pl.lo_bits;
       a.mask = (pl.passes == 2 && pass == 0) ? (uint32_t)((1 << pl.lo_bits) - 1) : 0xFFFFFFFFu;
       a.last = last ? 1 : 0;
       a.num_experts = (uint32_t)N;
-      a.top_k = num_experts_per_token;
-      const int64_t entries = (int64_t)a.bins * a.blocks;
-      const int scan_tiles = (int)((entries + kScanTile - 1) / kScanTile);
-      static std::atomic<uint64_t> configured{0};          // tables of up to 4 x 4097 counters exceed the 64 KiB default
-      if (hipError_t e = ensure_dynamic_lds((const void*)sort_scatter_kernel, kMaxBins * kSortWaves * 4, configured); e != hipSuccess)
-        return OMNI_ERR_HIP_BASE + (int)e;
-      hipLaunchKernelGGL(sort_count_kernel, dim3(a.blocks), dim3(kSortThreads), (size_t)a.bins * 4, s, a);
-      hipLaunchKernelGGL(scan_tiles_kernel, dim3(scan_tiles), dim3(kScanBlock), 0, s, hist, hist, tile_sums, entries);
-      hipLaunchKernelGGL(scan_fixup_kernel, dim3(scan_tiles), dim3(kScanBlock), 0, s, hist, (int32_t*)nullptr, tile_sums, entries, scan_tiles);
-      hipLaunchKernelGGL(sort_scatter_kernel, dim3(a.blocks), dim3(kSortThreads), (size_t)a.bins * kSortWaves * 4, s, a);
+      a.inv_top_k = num_experts_per_token > 0 ? ((1ull << 40) + num_experts_per_token - 1) / (uint64_t)num_experts_per_token : 0;
+      hipLaunchKernelGGL(sort_count_kernel, dim3(a.blocks), dim3(kSortThreads), (size_t)a.stride * 4, s, a);
+      hipLaunchKernelGGL(sort_scatter_kernel, dim3(a.blocks), dim3(kSortThreads), (size_t)a.stride * (kSortWaves + 1) * 4, s, a);
     }
-    sorted_keys = keys_b;
   }
-  const unsigned nb = (unsigned)((P + 256) / 256 < 2048 ? (P + 256) / 256 : 2048);
-  hipLaunchKernelGGL(segment_offsets_kernel, dim3(nb), dim3(256), 0, s, sorted_keys, offsets, P, (uint32_t)N);
+  if (!single) {
+    const int32_t* sorted_keys = P > 0 ? keys_b : indices;  // P == 0: nothing was sorted, every offset is 0
+    const unsigned nb = (unsigned)((P + 256) / 256 < 2048 ? (P + 256) / 256 : 2048);
+    hipLaunchKernelGGL(segment_offsets_kernel, dim3(nb), dim3(256), 0, s, sorted_keys, offsets, P, (uint32_t)N);
+  }
   hipError_t err = hipGetLastError();
   return err == hipSuccess ? OMNI_OK : OMNI_ERR_HIP_BASE + (int)err;
 }

@@ -81,7 +81,7 @@ def test_argument_errors_need_no_gpu():
     assert moe(8192, 64, 16, 4, 2) == -5         # rows beyond 8 KiB
     assert moe(64, 64, 16, 4, 2, dt=5) == -3
     assert lib.omni_mlp_fwd(p, p, p, p, None, p, 4, 64, 64, 0, None, None) == -6 # no workspace
-    assert lib.omni_schedule_workspace_bytes(4, 2, 100) >= 400
+    assert lib.omni_schedule_workspace_bytes(4, 2, 100) >= 200
 
 
 def test_ops_fail_loudly_without_gpu():

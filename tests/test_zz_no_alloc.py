@@ -53,8 +53,8 @@ def test_noalloc_schedule_two_pass_sort_and_limit(device):
     for w, h in zip(want, got):
         assert torch.equal(w, h)
     # beyond the fixed scratch: a clear error, nothing enqueued
-    T, k = 1 << 20, 16
-    assert lib.omni_schedule_workspace_bytes(T, k, 4096) > (8 << 20)
+    T, k = 1 << 20, 16                   # a two-pass sort of 16 Mi pairs keeps three arrays of them
+    assert lib.omni_schedule_workspace_bytes(T, k, N) > (8 << 20)
     p = idx.data_ptr()
-    assert lib.omni_schedule_noalloc(p, p, p, p, T, k, 4096, _lib.stream_ptr()) == -7
+    assert lib.omni_schedule_noalloc(p, p, p, p, T, k, N, _lib.stream_ptr()) == -7
     assert b"scratch" in lib.omni_error_string(-7)
