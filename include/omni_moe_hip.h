@@ -52,6 +52,7 @@ extern "C" {
 #define OMNI_EXPERT_ALGO_GATHER 1   /* token-resident gather, no schedule needed */
 #define OMNI_EXPERT_ALGO_SEGMENT 2  /* expert-centric segments from omni_schedule */
 #define OMNI_EXPERT_ALGO_SPLIT 3    /* hidden dimension cut into 8 slices, one per XCD: table slices stay in that XCD's L2 */
+#define OMNI_EXPERT_ALGO_DENSE 4    /* few experts, hundreds of tokens each: two MFMA GEMMs over all experts (the reference's group regime) */
 
 OMNI_API int32_t omni_abi_version(void);
 OMNI_API const char* omni_error_string(int32_t code);
@@ -115,6 +116,10 @@ OMNI_API int32_t omni_schedule_noalloc(const int32_t* indices, int32_t* offsets,
  *               omni_schedule, a pass over the sorted pairs for the coefficients, a token pass
  *               for the sum; kept so that the organisations can be measured side by side.
  *               GATHER and SEGMENT agree bit for bit, SPLIT to fp32 rounding of the dot products.
+ *               DENSE is for the regime of the reference's group path (omni_scheduler.py:58,103-226,
+ *               omni_expert.py:171-372: T*k/N > 256): a gate matrix G[T,N], C = silu(x U^T) * G on the matrix
+ *               cores (kept with 16 significant bits), y = C V on the matrix cores; bf16/f16, N % 32 == 0,
+ *               N <= 2048, H % 64 == 0.  AUTO takes it under the reference's rule where N <= 16 k.
  *   workspace : omni_expert_workspace_bytes() bytes for the same arguments (0 = may be NULL) */
 OMNI_API size_t omni_expert_workspace_bytes(int64_t num_tokens, int32_t hidden_size, int64_t num_experts,
                                    int32_t num_experts_per_token, int32_t dtype, int32_t algo);

@@ -25,6 +25,9 @@
 #include "omni_moe_hip.h"
 #include "rows.h"
 
+// gemm.hip: c[T, 2N] = [round(v) | round(v - round(v))], v = silu(x W^T) * gate
+int omni_gemm_gated(const void* x, const void* w, const float* gate, void* c, int64_t T, int64_t N, int64_t K, int dtype, void* stream);
+
 namespace omni {
 
 constexpr int kTokensPerBlock = 4;   // one wave each
@@ -438,11 +441,96 @@ static int expert_split_dispatch(const void* x, const void* up, const void* down
   return err == hipSuccess ? OMNI_OK : OMNI_ERR_HIP_BASE + (int)err;
 }
 
+// ---- dense variant ("dense" algorithm) --------------------------------------------------------
+// The regime of the reference's group path (omni_scheduler.py:58,103-226; omni_expert.py:171-372): so few experts
+// that each serves hundreds of tokens (T*k/N > 256).  The reference looks for 16 experts with identical token lists
+// and runs those through tl.dot; here the whole op becomes two MFMA GEMMs over ALL experts, which at this density
+// cost less than fetching 2k rows per token:
+//   G[t, e]  = sum of the gates of token t's slots that name expert e (0 elsewhere)      gate matrix, fp32
+//   C        = silu(x U^T) * G, kept as a 16-bit head and a 16-bit remainder [T, 2N]      GEMM with a gate epilogue
+//   y        = [C_head | C_rem] [V^T | V^T]^T                                             GEMM over K = 2N
+// silu and the gate product are fp32, C carries 16 significant bits, sums are fp32: results agree with the gather
+// algorithm to a few units of fp32 rounding of the coefficients.  Duplicate slots add their gates in slot order.
+constexpr int kDenseMaxExperts = 2048;
+
+// One wave per token: the token's row of G is built in LDS (slots in order, by one lane) and written out whole.
+__global__ __launch_bounds__(256) void dense_gate_rows_kernel(const void* __restrict__ gates, const int32_t* __restrict__ ids,
+                                                              float* __restrict__ gate_matrix, int num_tokens, int top_k,
+                                                              int num_experts, int dtype) {
+  extern __shared__ float rows[];                                  // [4 waves][num_experts]
+  const int lane = lane_id(), wave = threadIdx.x >> 6;
+  const int t = blockIdx.x * 4 + wave;
+  if (t >= num_tokens) return;
+  float* row = rows + wave * num_experts;
+  for (int e = lane; e < num_experts; e += kWave) row[e] = 0.f;
+  __builtin_amdgcn_wave_barrier();
+  if (lane == 0) {
+    for (int j = 0; j < top_k; ++j) {
+      const int id = ids[(int64_t)t * top_k + j];
+      if ((uint32_t)id < (uint32_t)num_experts) {
+        const float g = dtype == OMNI_BF16 ? Elem<kBF16>::load(gates, (int64_t)t * top_k + j) : Elem<kF16>::load(gates, (int64_t)t * top_k + j);
+        row[id] += g;
+      }
+    }
+  }
+  __builtin_amdgcn_wave_barrier();
+  for (int e = lane; e < num_experts; e += kWave) gate_matrix[(int64_t)t * num_experts + e] = row[e];
+}
+
+// vt2[h, c] = v[c % N, h] for c < 2N: the down table transposed, twice side by side (K-contiguous operand of the second GEMM)
+__global__ __launch_bounds__(256) void dense_transpose_kernel(const uint16_t* __restrict__ v, uint16_t* __restrict__ vt2, int num_experts, int hidden) {
+  __shared__ uint16_t tile[64][66];
+  const int e0 = blockIdx.x * 64, h0 = blockIdx.y * 64;
+  for (int i = threadIdx.x; i < 64 * 64; i += 256) {
+    const int e = i / 64, h = i % 64;
+    tile[e][h] = (e0 + e < num_experts && h0 + h < hidden) ? v[(int64_t)(e0 + e) * hidden + h0 + h] : (uint16_t)0;
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < 64 * 64; i += 256) {
+    const int h = i / 64, e = i % 64;
+    if (e0 + e < num_experts && h0 + h < hidden) {
+      const uint16_t x = tile[e][h];
+      vt2[(int64_t)(h0 + h) * 2 * num_experts + e0 + e] = x;
+      vt2[(int64_t)(h0 + h) * 2 * num_experts + num_experts + e0 + e] = x;
+    }
+  }
+}
+
+static inline bool dense_covers(int64_t T, int H, int64_t N, int k, int dtype) {
+  return dtype != OMNI_F32 && N % 32 == 0 && N <= kDenseMaxExperts && H % 64 == 0 && H % 8 == 0 && k > 0 && T > 0;
+}
+
+// workspace: gate matrix [T, N] f32 | coefficients [T, 2N] | transposed down table [H, 2N]
+static inline size_t dense_workspace_bytes(int64_t T, int H, int64_t N) {
+  return align256((size_t)T * N * 4) + align256((size_t)T * 2 * N * 2) + align256((size_t)H * 2 * N * 2);
+}
+
+static int expert_dense_dispatch(const void* x, const void* up, const void* down, const void* gates, const int32_t* ids, void* y,
+                                 int64_t T, int H, int k, int64_t N, int dtype, void* workspace, hipStream_t s) {
+  if (T == 0) return OMNI_OK;
+  if (!dense_covers(T, H, N, k, dtype)) return OMNI_ERR_UNSUPPORTED;
+  if (!workspace) return OMNI_ERR_WORKSPACE;
+  char* w = (char*)workspace;
+  float* gate_matrix = (float*)w;  w += align256((size_t)T * N * 4);
+  void* coef = w;                  w += align256((size_t)T * 2 * N * 2);
+  uint16_t* vt2 = (uint16_t*)w;
+  hipLaunchKernelGGL(dense_gate_rows_kernel, dim3((unsigned)((T + 3) / 4)), dim3(256), (size_t)4 * N * 4, s, gates, ids, gate_matrix, (int)T, k, (int)N, dtype);
+  hipLaunchKernelGGL(dense_transpose_kernel, dim3((unsigned)((N + 63) / 64), (unsigned)((H + 63) / 64)), dim3(256), 0, s,
+                     (const uint16_t*)down, vt2, (int)N, H);
+  if (hipError_t e = hipGetLastError(); e != hipSuccess) return OMNI_ERR_HIP_BASE + (int)e;
+  if (int e = omni_gemm_gated(x, up, gate_matrix, coef, T, N, H, dtype, s)) return e;
+  return omni_linear_fwd(coef, vt2, nullptr, y, T, (int32_t)(2 * N), H, dtype, s);
+}
+
 // What OMNI_EXPERT_ALGO_AUTO runs.  The split algorithm pays when the two tables overflow one
 // XCD's 4 MiB L2 while an eighth of them fits beside the streaming x and y rows, and when there
 // are enough pairs to amortise its second launch; otherwise rows are gathered whole.
 static int resolve_algo(int algo, int64_t T, int H, int64_t N, int k, int dtype) {
   if (algo != OMNI_EXPERT_ALGO_AUTO) return algo;
+  // the reference's rule for its group path (omni_scheduler.py:58, group_size 16): more than 256 pairs per expert --
+  // and no more than 16 experts per slot: the GEMMs cost N rows per token, the gather 2k (measured at 16384 tokens,
+  // hidden 1024: 66 us dense against 69 us gather at N = 256, k = 16; 95 against 70 at N = 512)
+  if (dense_covers(T, H, N, k, dtype) && T * (int64_t)k > 256 * N && N <= 16 * (int64_t)k) return OMNI_EXPERT_ALGO_DENSE;
   const int es = dtype == OMNI_F32 ? 4 : 2;
   const int64_t tables = 2 * N * (int64_t)H * es;
   const bool fits = split_lanes_per_row(H, es) != 0 && k <= 2 * kWave;
@@ -458,6 +546,8 @@ extern "C" OMNI_API size_t omni_expert_workspace_bytes(int64_t num_tokens, int32
   algo = omni::resolve_algo(algo, num_tokens, hidden_size, num_experts, num_experts_per_token, dtype);
   if (algo == OMNI_EXPERT_ALGO_SPLIT)
     return omni::align256((size_t)omni::kSlices * (size_t)num_tokens * (size_t)num_experts_per_token * 4);
+  if (algo == OMNI_EXPERT_ALGO_DENSE)
+    return omni::dense_covers(num_tokens, hidden_size, num_experts, num_experts_per_token, dtype) ? omni::dense_workspace_bytes(num_tokens, hidden_size, num_experts) : 0;
   if (algo != OMNI_EXPERT_ALGO_SEGMENT) return 0;   // the gather algorithm keeps everything in registers
   const size_t P = (size_t)num_tokens * (size_t)num_experts_per_token;
   return omni::align256((size_t)(num_experts + 1) * 4) + 2 * omni::align256(P * 4) +
@@ -491,6 +581,13 @@ extern "C" OMNI_API int32_t omni_expert_fwd(const void* x, const void* up_weight
       case OMNI_F32: return expert_split_dispatch<kF32>(x, up_weight, down_weight, routing_weights, indices, y, num_tokens, hidden_size, num_experts_per_token, num_experts, workspace, s);
       default: return OMNI_ERR_DTYPE;
     }
+  }
+  if (algo == OMNI_EXPERT_ALGO_DENSE) {
+    if (dtype != OMNI_BF16 && dtype != OMNI_F16 && dtype != OMNI_F32) return OMNI_ERR_DTYPE;
+    if (num_experts_per_token == 0)   // writes zeros
+      return omni_expert_fwd(x, up_weight, down_weight, routing_weights, indices, y, num_tokens, hidden_size, num_experts, 0, dtype, OMNI_EXPERT_ALGO_GATHER, nullptr, stream);
+    return expert_dense_dispatch(x, up_weight, down_weight, routing_weights, indices, y, num_tokens, hidden_size, num_experts_per_token,
+                                 num_experts, dtype, workspace, s);
   }
   if (algo != OMNI_EXPERT_ALGO_GATHER) return OMNI_ERR_UNSUPPORTED;
   switch (dtype) {

@@ -33,7 +33,7 @@ constexpr int kBK = 64;                       // K elements per LDS stage
 constexpr int kRowBytes = kBK * 2 + 16;       // padded LDS row
 constexpr int kGemmThreads = 256;
 
-enum : int { kEpiPlain = 0, kEpiSwiglu = 1, kEpiResidual = 2, kEpiStats = 3 };   // kEpiStats: plain + column statistics
+enum : int { kEpiPlain = 0, kEpiSwiglu = 1, kEpiResidual = 2, kEpiStats = 3, kEpiGate = 4 };   // kEpiStats: plain + column statistics; kEpiGate: silu(acc) * gate, as a pair of 16-bit values
 
 template <int DT> struct ElemBytes { static constexpr int value = (DT == kF32) ? 4 : 2; };
 
@@ -76,6 +76,7 @@ struct GemmArgs {           // all element offsets below are scaled by the eleme
   int single;             // N % 4 != 0: rows are not 8-byte aligned, results leave element by element
   float* part_mean;       // kEpiStats only: [ceil(M/32)][N] mean of each column over
   float* part_m2;         //   rows 32s..32s+31 of the ROUNDED result, and the sum of squared deviations
+  const float* gate;      // kEpiGate only: [M, N] fp32 factors; C is then [M, 2N]: round(v) in columns 0..N-1, round(v - round(v)) in N..2N-1
 };
 
 // Which output tile a block owns.  Blocks go round-robin over the 8 XCDs; each XCD gets
@@ -202,6 +203,37 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, f32x16_t (&acc)
 #pragma unroll
           for (int pr = 0; pr < 2; ++pr) {
             if (nt + pr * 16 >= g.N) continue;             // same answer in both lanes of a pair
+            if constexpr (EPI == kEpiGate) {
+              // c = silu(acc) * gate in fp32, stored as a 16-bit head and a 16-bit remainder (head + remainder carries 16
+              // significant bits), so that a following GEMM over [head | remainder] sums in nearly full precision
+              uint32_t hw[2][2], lw[2][2];
+#pragma unroll
+              for (int e = 0; e < 2; ++e) {
+                const int q4 = 2 * pr + e;
+                const int n = nt + q4 * 8 + (lane >> 5) * 4;
+                f32x4_t gt = {0.f, 0.f, 0.f, 0.f};
+                if (n < g.N) gt = *(const f32x4_t*)(g.gate + (int64_t)m * g.N + n);
+                float hv[4], lv[4];
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                  const float c = silu_f32(acc[i][j][q4 * 4 + q]) * gt[q];
+                  hv[q] = Elem<DT>::round(c);
+                  lv[q] = c - hv[q];
+                }
+                hw[e][0] = pack2<DT>(hv[0], hv[1]); hw[e][1] = pack2<DT>(hv[2], hv[3]);
+                lw[e][0] = pack2<DT>(lv[0], lv[1]); lw[e][1] = pack2<DT>(lv[2], lv[3]);
+              }
+              const auto h0 = __builtin_amdgcn_permlane32_swap(hw[0][0], hw[1][0], false, false);
+              const auto h1 = __builtin_amdgcn_permlane32_swap(hw[0][1], hw[1][1], false, false);
+              const auto l0 = __builtin_amdgcn_permlane32_swap(lw[0][0], lw[1][0], false, false);
+              const auto l1 = __builtin_amdgcn_permlane32_swap(lw[0][1], lw[1][1], false, false);
+              const int n = nt + pr * 16 + (lane >> 5) * 8;
+              if (n < g.N) {
+                *(u32x4_t*)(g.c + ((int64_t)m * 2 * g.N + n) * 2) = u32x4_t{h0[0], h1[0], h0[1], h1[1]};
+                *(u32x4_t*)(g.c + ((int64_t)m * 2 * g.N + g.N + n) * 2) = u32x4_t{l0[0], l1[0], l0[1], l1[1]};
+              }
+              continue;
+            }
             uint32_t w[2][2];
 #pragma unroll
             for (int e = 0; e < 2; ++e) {
@@ -590,6 +622,7 @@ static hipError_t launch_gemm(GemmArgs g, hipStream_t s) {
   g.patch_m = g.patch_n = 0;
   g.wide = (DT != kF32) && g.N % 8 == 0 && ((uintptr_t)g.c % 16 == 0);
   g.single = g.N % 4 != 0;
+  if (EPI == kEpiGate && !(g.wide && (uintptr_t)g.gate % 16 == 0)) return hipErrorInvalidValue;   // the gate epilogue has the 16-byte form only
   if (blocks % 256 == 0) {
     if (g.tiles_m % 4 == 0 && g.tiles_n % 8 == 0) { g.patch_m = 4; g.patch_n = 8; }
     else if (g.tiles_m % 8 == 0 && g.tiles_n % 4 == 0) { g.patch_m = 8; g.patch_n = 4; }
@@ -629,7 +662,7 @@ static int gemm_plain(const void* a, const void* b, const void* b_hi, const void
                       float* part_mean = nullptr, float* part_m2 = nullptr) {
   if (int e = check_gemm(M, N, K, ElemBytes<DT>::value)) return e;
   if (M == 0) return OMNI_OK;
-  GemmArgs g{(const uint8_t*)a, (const uint8_t*)b, (const uint8_t*)b_hi, (const uint8_t*)res, (uint8_t*)c, (int)M, (int)N, (int)K, 0, 0, 0, 0, 0, 0, nullptr, nullptr};
+  GemmArgs g{(const uint8_t*)a, (const uint8_t*)b, (const uint8_t*)b_hi, (const uint8_t*)res, (uint8_t*)c, (int)M, (int)N, (int)K, 0, 0, 0, 0, 0, 0, nullptr, nullptr, nullptr};
   g.part_mean = part_mean;
   g.part_m2 = part_m2;
   const int64_t big = ((M + 255) / 256) * ((N + 255) / 256), mid = ((M + 127) / 128) * ((N + 127) / 128);
@@ -654,7 +687,7 @@ template <int DT>
 static int gemm_swiglu(const void* x, const void* wg, const void* wu, void* h, int64_t M, int64_t I, int64_t K, hipStream_t s) {
   if (int e = check_gemm(M, I, K, ElemBytes<DT>::value)) return e;
   if (M == 0) return OMNI_OK;
-  GemmArgs g{(const uint8_t*)x, (const uint8_t*)wg, (const uint8_t*)wu, nullptr, (uint8_t*)h, (int)M, (int)I, (int)K, 0, 0, 0, 0, 0, 0, nullptr, nullptr};
+  GemmArgs g{(const uint8_t*)x, (const uint8_t*)wg, (const uint8_t*)wu, nullptr, (uint8_t*)h, (int)M, (int)I, (int)K, 0, 0, 0, 0, 0, 0, nullptr, nullptr, nullptr};
   const int64_t big = ((M + 255) / 256) * ((I + 127) / 128);
   hipError_t err;
   if (big >= 200) err = launch_gemm<DT, 4, 4, kEpiSwiglu>(g, s);
@@ -663,6 +696,28 @@ static int gemm_swiglu(const void* x, const void* wg, const void* wu, void* h, i
 }
 
 }  // namespace omni
+
+// c[T, 2N] = [round(v) | round(v - round(v))] with v = silu(x W^T) * gate, gate [T, N] fp32 (16-bit storage types only)
+int omni_gemm_gated(const void* x, const void* w, const float* gate, void* c, int64_t T, int64_t N, int64_t K, int dtype, void* stream) {
+  using namespace omni;
+  if (dtype != OMNI_BF16 && dtype != OMNI_F16) return OMNI_ERR_UNSUPPORTED;
+  if (int e = check_gemm(T, N, K, 2)) return e;
+  if (T == 0) return OMNI_OK;
+  GemmArgs g{(const uint8_t*)x, (const uint8_t*)w, nullptr, nullptr, (uint8_t*)c, (int)T, (int)N, (int)K, 0, 0, 0, 0, 0, 0, nullptr, nullptr, gate};
+  hipStream_t s = (hipStream_t)stream;
+  const int64_t big = ((T + 255) / 256) * ((N + 255) / 256), mid = ((T + 127) / 128) * ((N + 127) / 128);
+  hipError_t err;
+  if (dtype == OMNI_BF16) {
+    if (big >= 200) err = launch_gemm<kBF16, 4, 4, kEpiGate>(g, s);
+    else if (mid >= 200) err = launch_gemm<kBF16, 2, 2, kEpiGate>(g, s);
+    else err = launch_gemm<kBF16, 1, 1, kEpiGate>(g, s);
+  } else {
+    if (big >= 200) err = launch_gemm<kF16, 4, 4, kEpiGate>(g, s);
+    else if (mid >= 200) err = launch_gemm<kF16, 2, 2, kEpiGate>(g, s);
+    else err = launch_gemm<kF16, 1, 1, kEpiGate>(g, s);
+  }
+  return to_code(err);
+}
 
 int omni_gemm_router_projection(const void* x, const void* wx, const void* wy, void* z, float* part_mean, float* part_m2,
                                 int64_t T, int H, int r, int dtype, void* stream) {

@@ -17,7 +17,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libomni_moe_hip.so")
 
 OMNI_BF16, OMNI_F16, OMNI_F32 = 0, 1, 2
-ALGO_AUTO, ALGO_GATHER, ALGO_SEGMENT, ALGO_SPLIT = 0, 1, 2, 3
+ALGO_AUTO, ALGO_GATHER, ALGO_SEGMENT, ALGO_SPLIT, ALGO_DENSE = 0, 1, 2, 3, 4
 ERR_TOPK, ERR_SHAPE = -4, -2
 
 DTYPE_CODE = {torch.bfloat16: OMNI_BF16, torch.float16: OMNI_F16, torch.float32: OMNI_F32}

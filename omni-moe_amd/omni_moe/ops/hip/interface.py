@@ -139,7 +139,7 @@ def hip_omni_schedule_func(indices: torch.Tensor, num_experts: int) -> Schedule:
     return Schedule(offsets, pair_ids, token_ids)
 
 
-_ALGOS = {"auto": _lib.ALGO_AUTO, "gather": _lib.ALGO_GATHER, "segment": _lib.ALGO_SEGMENT, "split": _lib.ALGO_SPLIT}
+_ALGOS = {"auto": _lib.ALGO_AUTO, "gather": _lib.ALGO_GATHER, "segment": _lib.ALGO_SEGMENT, "split": _lib.ALGO_SPLIT, "dense": _lib.ALGO_DENSE}
 
 
 def hip_omni_expert_func(

@@ -234,6 +234,64 @@ def test_expert_split_algorithm(case, device):
     assert (got.float() - ref).abs().max().item() <= (1e-2 if dtype != torch.float32 else 1e-5) * scale
 
 
+DENSE_CASES = [(16384, 1024, 256, 16, torch.bfloat16, "baseline"),   # the shape the build plan names for the group regime: 1024 pairs per expert
+               (4096, 512, 64, 8, torch.bfloat16, "ref"),              # negative gates, ids with replacement (duplicates add)
+               (2048, 256, 32, 6, torch.float16, "ref"),
+               (1000, 1024, 96, 10, torch.bfloat16, "ref"),            # ragged token count, N a multiple of 32 only
+               (333, 64, 2048, 4, torch.bfloat16, "ref")]              # sparse use of the largest table the algorithm takes
+
+
+@pytest.mark.parametrize("case", DENSE_CASES, ids=lambda c: f"T{c[0]}-H{c[1]}-N{c[2]}-k{c[3]}-{str(c[4]).split('.')[-1]}-{c[5]}")
+def test_expert_dense_algorithm(case, device):
+    """The dense organisation for the reference's group regime (T*k/N > 256, omni_scheduler.py:58): a gate matrix and two
+    MFMA GEMMs over all experts.  Same tolerance against the oracle; agreement with the gather algorithm to the 16
+    significant bits its coefficients carry; run-to-run identical; AUTO picks it under the reference's rule where the
+    experts are few enough (N <= 16 k)."""
+    from omni_moe.ops.hip import _lib
+    T, H, N, k, dtype, kind = case
+    x, up, down, gates, ids = _expert_inputs(T, H, N, k, dtype, kind, seed=T + H)
+    d = [t.to(device) for t in (x, up, down, gates, ids)]
+    print(f"expert dense T={T} H={H} N={N} k={k} {dtype} {kind}", flush=True)
+    got = _ops().hip_omni_expert_func(*d, algo="dense")
+    assert torch.equal(got, _ops().hip_omni_expert_func(*d, algo="dense"))
+    want = oracle.expert_forward(x, up, down, gates, ids)
+    torch.testing.assert_close(got.cpu().float(), want.float(), **_tol(dtype))
+    ref = _ops().hip_omni_expert_func(*d, algo="gather").float()
+    scale = max(ref.abs().max().item(), 1e-6)
+    assert (got.float() - ref).abs().max().item() <= 1e-2 * scale          # one storage ulp where the sums straddle a rounding boundary
+    assert (got.float() != ref).float().mean().item() < 0.05
+    lib = _lib.load()
+    auto_ws = lib.omni_expert_workspace_bytes(T, H, N, k, _lib.DTYPE_CODE[dtype], _lib.ALGO_AUTO)
+    dense_ws = lib.omni_expert_workspace_bytes(T, H, N, k, _lib.DTYPE_CODE[dtype], _lib.ALGO_DENSE)
+    picks = T * k > 256 * N and N <= 16 * k              # the reference's group rule, and few enough experts for the GEMMs to pay
+    assert dense_ws > 0 and (auto_ws == dense_ws) == picks
+    if picks:
+        assert torch.equal(_ops().hip_omni_expert_func(*d), got)
+
+
+def test_expert_dense_refusals_and_bad_ids(device):
+    hip = _ops()
+    x, up, down, gates, ids = (t.to(device) for t in _expert_inputs(64, 128, 48, 4, torch.bfloat16, "ref", 3))
+    with pytest.raises(ValueError):                       # 48 experts: not a multiple of 32
+        hip.hip_omni_expert_func(x, up, down, gates, ids, algo="dense")
+    x, up, down, gates, ids = (t.to(device) for t in _expert_inputs(64, 128, 64, 4, torch.float32, "ref", 3))
+    with pytest.raises(ValueError):                       # fp32 storage
+        hip.hip_omni_expert_func(x, up, down, gates, ids, algo="dense")
+    g = torch.Generator().manual_seed(5)
+    T, H, N, k = 3000, 512, 128, 8
+    x, up, down = torch.randn(T, H, generator=g).bfloat16(), (torch.randn(N, H, generator=g) * 0.05).bfloat16(), (torch.randn(N, H, generator=g) * 0.05).bfloat16()
+    gates = torch.rand(T, k, generator=g).bfloat16()
+    ids = torch.randint(0, N, (T, k), generator=g, dtype=torch.int32)
+    ids[::7, 3] = N + 5                                    # ids outside the table contribute nothing
+    ids[::11, 0] = -1
+    ok = (ids >= 0) & (ids < N)
+    want = oracle.expert_forward(x, up, down, torch.where(ok, gates, torch.zeros_like(gates)), torch.where(ok, ids, torch.zeros_like(ids)))
+    got = hip.hip_omni_expert_func(*(t.to(device) for t in (x, up, down, gates, ids)), algo="dense")
+    torch.testing.assert_close(got.cpu().float(), want.float(), rtol=2e-2, atol=2e-2)
+    y0 = hip.hip_omni_expert_func(x.to(device), up.to(device), down.to(device), gates[:, :0].to(device), ids[:, :0].to(device), algo="dense")
+    assert torch.count_nonzero(y0).item() == 0             # k = 0 -> zeros
+
+
 def test_expert_split_bad_ids(device):
     g = torch.Generator().manual_seed(12)
     T, H, N, k = 2100, 1024, 512, 8
