@@ -242,7 +242,10 @@ OMNI_API int32_t omni_linear2_fwd(const void* x, const void* weight_lo, const vo
  *   running_mean_*, running_var_* [r] of dtype stats_dtype; num_batches_tracked_* int64
  *     scalars (may be NULL).  training != 0: batch statistics normalise (biased variance)
  *     and the buffers are UPDATED in place with `momentum` (unbiased variance), as
- *     nn.BatchNorm1d in train mode; training == 0: the buffers normalise, nothing is written.
+ *     nn.BatchNorm1d in train mode; momentum < 0 stands for momentum=None, the cumulative
+ *     average with factor 1 / num_batches_tracked (the counters are then required); one token in
+ *     training is OMNI_ERR_SHAPE (nn.BatchNorm1d raises).  training == 0: the buffers
+ *     normalise, nothing is written.
  *   gates [T,k] dtype = exp(score); indices [T,k] int32; scores [T,k] dtype or NULL
  *   workspace: omni_router_workspace_bytes() bytes */
 OMNI_API size_t omni_router_workspace_bytes(int64_t num_tokens, int32_t num_expert_sqrt, int32_t dtype);

@@ -45,6 +45,7 @@ extern "C" OMNI_API int32_t omni_moe_fwd(const void* x, const void* gate_weight,
     if (r * r > num_experts) return OMNI_ERR_SHAPE;                                                   // ids reach r*r - 1
   }
   if (num_tokens == 0) return OMNI_OK;
+  if (training && num_tokens == 1) return OMNI_ERR_SHAPE;   // batch statistics of one sample: nn.BatchNorm1d raises
   if (!x || !y || !up_embed || !down_embed) return OMNI_ERR_NULL;
   if (!workspace) return OMNI_ERR_WORKSPACE;
   if (side_stream && (!fork_event || !join_event)) return OMNI_ERR_NULL;

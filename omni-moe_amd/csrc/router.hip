@@ -211,7 +211,16 @@ struct SelectArgs {
   int32_t* indices;      // [T,k]
   int num_tokens, r, k, kp, dt;
   uint8_t row_cells[128]; // candidate cells in row a: min(kp, k/(a+1)), filled by select_dispatch
+  int64_t* count_batch[2]; // NULL, or BatchNorm's num_batches_tracked of the two halves: incremented here, behind the
+                           // kernel that read them (train-mode router stage)
 };
+
+__device__ __forceinline__ void count_batch(const SelectArgs& g) {
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    if (g.count_batch[0]) *g.count_batch[0] += 1;
+    if (g.count_batch[1]) *g.count_batch[1] += 1;
+  }
+}
 
 // BatchNorm (affine-free) then log-softmax of one half, in place: v holds the raw projection
 // of key a*64+lane (NaN-free -inf padding past r).  Each stage rounds to the storage dtype
@@ -238,6 +247,7 @@ __device__ __forceinline__ void normalise_half(float (&v)[R], const float* mean,
 // R = half keys per lane (r <= 64*R); C = candidate cells per lane.
 template <int R, int C>
 __global__ __launch_bounds__(kRouterWaves* kWave) void router_select_kernel(const SelectArgs g) {
+  count_batch(g);
   const int lane = lane_id();
   const int wave = blockIdx.x * kRouterWaves + (threadIdx.x >> 6);
   const int num_waves = gridDim.x * kRouterWaves;
@@ -401,6 +411,7 @@ __device__ __forceinline__ uint32_t sorted_key(const uint32_t (&v)[R], int i) {
 // Same selection as router_select_kernel for bf16 / f16 storage, on packed keys.
 template <int R, int C>
 __global__ __launch_bounds__(kRouterWaves* kWave) void router_select_packed_kernel(const SelectArgs g) {
+  count_batch(g);
   const int lane = lane_id();
   const int wave = blockIdx.x * kRouterWaves + (threadIdx.x >> 6);
   const int num_waves = gridDim.x * kRouterWaves;
@@ -519,9 +530,10 @@ struct BnFinalArgs {
   float* stats;             // [4][r]: mean_x, rstd_x, mean_y, rstd_y
   void* running_mean[2];    // [r] each, dtype stat_dt; read in eval, updated in training
   void* running_var[2];
-  int64_t* num_batches_tracked[2];   // may be NULL
+  int64_t* num_batches_tracked[2];   // may be NULL; read for the cumulative average (momentum < 0)
   int num_rows, r, strips, training, stat_dt;
-  float momentum, eps;
+  int count_here;                    // increment num_batches_tracked in this kernel (no select kernel follows; momentum >= 0 only)
+  float momentum, eps;               // momentum < 0: cumulative moving average, factor 1 / (batches tracked so far + 1)
 };
 
 __device__ __forceinline__ double wave_sum_f64(double v) {
@@ -536,7 +548,7 @@ __device__ __forceinline__ double wave_sum_f64(double v) {
 // the running buffers provide mean and variance.
 __global__ __launch_bounds__(256) void bn_finalize_kernel(const BnFinalArgs g) {
   const int col = blockIdx.x * (256 / kWave) + (threadIdx.x >> 6), lane = lane_id();
-  if (col == 0 && lane == 0 && g.training) {
+  if (col == 0 && lane == 0 && g.training && g.count_here) {
     if (g.num_batches_tracked[0]) *g.num_batches_tracked[0] += 1;
     if (g.num_batches_tracked[1]) *g.num_batches_tracked[1] += 1;
   }
@@ -559,8 +571,10 @@ __global__ __launch_bounds__(256) void bn_finalize_kernel(const BnFinalArgs g) {
     if (lane == 0) {
       const float unbiased = (float)(m2 / (n > 1. ? n - 1. : 1.));
       const float rm = load_score(g.running_mean[half], key, g.stat_dt), rv = load_score(g.running_var[half], key, g.stat_dt);
-      store_score(g.running_mean[half], key, (1.f - g.momentum) * rm + g.momentum * mean, g.stat_dt);
-      store_score(g.running_var[half], key, (1.f - g.momentum) * rv + g.momentum * unbiased, g.stat_dt);
+      // nn.BatchNorm1d(momentum=None): the factor is 1 / num_batches_tracked AFTER this batch has been counted
+      const float f = g.momentum >= 0.f ? g.momentum : 1.0f / (float)(*g.num_batches_tracked[half] + 1);
+      store_score(g.running_mean[half], key, (1.f - f) * rm + f * mean, g.stat_dt);
+      store_score(g.running_var[half], key, (1.f - f) * rv + f * unbiased, g.stat_dt);
     }
   } else {
     mean = load_score(g.running_mean[half], key, g.stat_dt);
@@ -586,7 +600,7 @@ extern "C" OMNI_API int32_t omni_router_select(const void* logits_x, const void*
   if (dtype != OMNI_BF16 && dtype != OMNI_F16 && dtype != OMNI_F32) return OMNI_ERR_DTYPE;
   if (num_tokens == 0 || k == 0) return OMNI_OK;
   if (!logits_x || !logits_y || !scores || !indices) return OMNI_ERR_NULL;
-  SelectArgs g{logits_x, logits_y, r, nullptr, scores, nullptr, indices, (int)num_tokens, r, k, 0, dtype};
+  SelectArgs g{logits_x, logits_y, r, nullptr, scores, nullptr, indices, (int)num_tokens, r, k, 0, dtype, {}, {nullptr, nullptr}};
   return select_dispatch(g, (hipStream_t)stream);
 }
 
@@ -622,7 +636,10 @@ extern "C" OMNI_API int32_t omni_router_fwd(const void* x, const void* weight_x,
   if (dtype != OMNI_BF16 && dtype != OMNI_F16 && dtype != OMNI_F32) return OMNI_ERR_DTYPE;
   if (stats_dtype != OMNI_BF16 && stats_dtype != OMNI_F16 && stats_dtype != OMNI_F32) return OMNI_ERR_DTYPE;
   if (num_tokens == 0) return OMNI_OK;
+  if (training && num_tokens == 1) return OMNI_ERR_SHAPE;   // batch statistics of one sample: nn.BatchNorm1d raises
   if (!x || !weight_x || !weight_y || !running_mean_x || !running_var_x || !running_mean_y || !running_var_y) return OMNI_ERR_NULL;
+  if (training && momentum < 0.f && (!num_batches_tracked_x || !num_batches_tracked_y)) return OMNI_ERR_NULL;   // the cumulative average needs the counts
+  if (training && momentum < 0.f && k == 0) return OMNI_ERR_UNSUPPORTED;
   if (k > 0 && (!gates || !indices)) return OMNI_ERR_NULL;
   if (!workspace) return OMNI_ERR_WORKSPACE;
   hipStream_t s = (hipStream_t)stream;
@@ -640,11 +657,12 @@ extern "C" OMNI_API int32_t omni_router_fwd(const void* x, const void* weight_x,
                                           num_tokens, hidden_size, r, dtype, stream)) return e;
   BnFinalArgs b{part_mean, part_m2, stats, {running_mean_x, running_mean_y}, {running_var_x, running_var_y},
                 {num_batches_tracked_x, num_batches_tracked_y}, (int)num_tokens, r, (int)strips, training ? 1 : 0, stats_dtype,
-                momentum, eps};
+                k == 0 ? 1 : 0, momentum, eps};
   hipLaunchKernelGGL(bn_finalize_kernel, dim3((2 * r + 3) / 4), dim3(256), 0, s, b);
   hipError_t err = hipGetLastError();
   if (err != hipSuccess) return OMNI_ERR_HIP_BASE + (int)err;
   if (k == 0) return OMNI_OK;
-  SelectArgs g{z, (const char*)z + (size_t)r * es, 2 * r, stats, scores, gates, indices, (int)num_tokens, r, k, 0, dtype};
+  SelectArgs g{z, (const char*)z + (size_t)r * es, 2 * r, stats, scores, gates, indices, (int)num_tokens, r, k, 0, dtype, {},
+               {training ? num_batches_tracked_x : nullptr, training ? num_batches_tracked_y : nullptr}};
   return select_dispatch(g, s);
 }

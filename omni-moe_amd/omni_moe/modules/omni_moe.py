@@ -69,11 +69,16 @@ class OmniMoE(nn.Module):
     def act_fn(self, x: torch.Tensor) -> torch.Tensor:
         return torch.nn.functional.silu(x)
 
+    def _router_norms(self):
+        """The two BatchNorm modules; the library applies one momentum and one eps to both halves."""
+        nx, ny = self.router_norm_x, self.router_norm_y
+        if nx.momentum != ny.momentum or nx.eps != ny.eps:
+            raise ValueError("router_norm_x and router_norm_y must share momentum and eps")
+        return nx, ny
+
     def route(self, hidden_states: torch.Tensor, return_scores: bool = False):
         """Router only: (gates, indices[, scores]) for ``[tokens, hidden]`` input."""
-        nx, ny = self.router_norm_x, self.router_norm_y
-        if nx.momentum is None or ny.momentum is None:
-            raise NotImplementedError("cumulative-average BatchNorm (momentum=None) is not covered")
+        nx, ny = self._router_norms()
         return hip_omni_router_fwd_func(
             hidden_states, self.router_gate_x.weight, self.router_gate_y.weight,
             nx.running_mean, nx.running_var, nx.num_batches_tracked,
@@ -113,11 +118,9 @@ class OmniMoE(nn.Module):
 
     def forward(self, hidden_states: torch.Tensor, **kwargs) -> torch.Tensor:
         bsz, seq_len, _ = hidden_states.shape
-        nx, ny = self.router_norm_x, self.router_norm_y
         if torch.is_grad_enabled() and (hidden_states.requires_grad or any(p.requires_grad for p in self.parameters())):
             return self._forward_differentiable(hidden_states)
-        if nx.momentum is None or ny.momentum is None:
-            raise NotImplementedError("cumulative-average BatchNorm (momentum=None) is not covered")
+        nx, ny = self._router_norms()
         with torch.no_grad():
             x = hidden_states.view(-1, self.hidden_size)
             two = (self.overlap_branches and x.is_cuda

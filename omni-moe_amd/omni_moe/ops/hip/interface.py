@@ -434,6 +434,8 @@ def hip_omni_router_fwd_func(
     for nbt in (num_batches_tracked_x, num_batches_tracked_y):
         if nbt is not None and (nbt.dtype != torch.int64 or nbt.numel() != 1):
             raise TypeError("num_batches_tracked must be an int64 scalar tensor")
+    _check_batch_norm_call(x.size(0), r, training, momentum, num_batches_tracked_x, num_batches_tracked_y)
+    momentum = -1.0 if momentum is None else momentum
     _lib.require_gpu(x, weight_x, weight_y, *stats)
     if _needs_grad(x, weight_x, weight_y):
         if return_scores:
@@ -444,6 +446,14 @@ def hip_omni_router_fwd_func(
     out = _router_stage_forward(x, weight_x, weight_y, running_mean_x, running_var_x, num_batches_tracked_x,
                                 running_mean_y, running_var_y, num_batches_tracked_y, k, training, momentum, eps, return_scores)
     return out[:3] if return_scores else out[:2]
+
+
+def _check_batch_norm_call(num_tokens, r, training, momentum, nbt_x, nbt_y):
+    """What nn.BatchNorm1d checks itself (reference omni_moe.py:53-54,70-71)."""
+    if training and num_tokens == 1:
+        raise ValueError(f"Expected more than 1 value per channel when training, got input size torch.Size([1, {r}])")
+    if training and momentum is None and (nbt_x is None or nbt_y is None):
+        raise ValueError("momentum=None (cumulative moving average) needs num_batches_tracked")
 
 
 def _router_stage_forward(x, weight_x, weight_y, running_mean_x, running_var_x, num_batches_tracked_x,
@@ -540,6 +550,8 @@ def hip_omni_moe_fwd_func(
     assert 0 <= k <= r * r, f"num_experts_per_token should be in [0, {r * r}], but got {k}"
     assert k <= 128, "num_experts_per_token should be less than or equal to 128"
     assert k % 2 == 0, "num_experts_per_token should be a multiple of 2"
+    _check_batch_norm_call(T, r, training, momentum, num_batches_tracked_x, num_batches_tracked_y)
+    momentum = -1.0 if momentum is None else momentum
     dev = _lib.require_gpu(x, *weights, *stats)
     x = _c(x)
     lib = _lib.load()

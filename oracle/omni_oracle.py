@@ -83,20 +83,28 @@ def batch_norm(
     running_mean: torch.Tensor,
     running_var: torch.Tensor,
     training: bool,
-    momentum: float = BN_MOMENTUM,
+    momentum: Optional[float] = BN_MOMENTUM,
     eps: float = BN_EPS,
     update: bool = True,
+    num_batches_tracked: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
     """``nn.BatchNorm1d(r, affine=False)`` on ``[T, r]`` (reference omni_moe.py:53-54,70-71).
 
     Train: batch mean and *biased* variance over the T rows normalise; the
     buffers move by ``momentum`` towards the batch mean and the *unbiased*
     variance.  Eval: the buffers normalise.  Statistics are fp32 whatever the
-    storage dtype; the result is rounded once to z's dtype.
+    storage dtype; the result is rounded once to z's dtype.  ``momentum=None`` is the
+    module's cumulative moving average: the factor is 1 / (batches tracked so far + 1),
+    read from ``num_batches_tracked`` (which the caller increments afterwards).  One sample
+    in training raises, as the module does.
     """
     zf = z.float()
     if training:
         T = zf.size(0)
+        if T == 1:
+            raise ValueError(f"Expected more than 1 value per channel when training, got input size {tuple(z.shape)}")
+        if momentum is None:
+            momentum = 1.0 / (float(num_batches_tracked) + 1.0)
         mean = zf.mean(0)
         var = ((zf - mean) ** 2).mean(0)
         if update:
@@ -129,7 +137,7 @@ class BNState:
 
 def router_forward(
     x: torch.Tensor, wx: torch.Tensor, wy: torch.Tensor,
-    bn_x: BNState, bn_y: BNState, top_k: int, training: bool,
+    bn_x: BNState, bn_y: BNState, top_k: int, training: bool, momentum: Optional[float] = BN_MOMENTUM,
 ):
     """Projection -> BN -> log-softmax -> select -> exp (reference omni_moe.py:147-178).
 
@@ -138,8 +146,8 @@ def router_forward(
     """
     r = wx.size(0)
     zx, zy = x @ wx.t(), x @ wy.t()
-    nx = batch_norm(zx, bn_x.running_mean, bn_x.running_var, training)
-    ny = batch_norm(zy, bn_y.running_mean, bn_y.running_var, training)
+    nx = batch_norm(zx, bn_x.running_mean, bn_x.running_var, training, momentum, num_batches_tracked=bn_x.num_batches_tracked)
+    ny = batch_norm(zy, bn_y.running_mean, bn_y.running_var, training, momentum, num_batches_tracked=bn_y.num_batches_tracked)
     if training:
         bn_x.num_batches_tracked += 1
         bn_y.num_batches_tracked += 1
@@ -229,12 +237,12 @@ class MoEWeights:
 
 def moe_forward(
     hidden_states: torch.Tensor, w: MoEWeights, bn_x: BNState, bn_y: BNState,
-    top_k: int, training: bool, expert_compute_dtype=torch.float32,
+    top_k: int, training: bool, expert_compute_dtype=torch.float32, momentum: Optional[float] = BN_MOMENTUM,
 ):
     """Whole layer (reference omni_moe.py:139-194).  Returns (y, gates, ids)."""
     shp = hidden_states.shape
     x = hidden_states.reshape(-1, shp[-1])
-    gates, ids, _ = router_forward(x, w.router_gate_x, w.router_gate_y, bn_x, bn_y, top_k, training)
+    gates, ids, _ = router_forward(x, w.router_gate_x, w.router_gate_y, bn_x, bn_y, top_k, training, momentum)
     e = expert_forward(x, w.up_embed, w.down_embed, gates, ids, compute_dtype=expert_compute_dtype)
     m = mlp_forward(x, w.gate_proj, w.up_proj, w.down_proj)
     return (m + e).reshape(shp), gates, ids

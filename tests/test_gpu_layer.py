@@ -407,6 +407,33 @@ def test_layer_is_graph_capturable(overlap, device):
         torch.cuda.synchronize()
 
 
+def test_layer_cumulative_batch_norm(device):
+    """router_norm_x/y with momentum=None (cumulative moving average, factor 1 / num_batches_tracked): three training
+    steps on different batches leave the buffers the oracle predicts, counters included."""
+    from omni_moe.modules.omni_moe import OmniMoE, OmniMoEConfig
+    T, H, I, N, k = 300, 128, 256, 256, 8
+    _, w = oracle.make_layer_inputs(9, T, H, I, N, dtype=torch.float32)
+    layer = OmniMoE(OmniMoEConfig(H, I, "silu", N, k))
+    layer.router_norm_x.momentum = layer.router_norm_y.momentum = None
+    layer.load_state_dict({"gate_proj.weight": w.gate_proj, "up_proj.weight": w.up_proj, "down_proj.weight": w.down_proj,
+                           "router_gate_x.weight": w.router_gate_x, "router_gate_y.weight": w.router_gate_y,
+                           "up_embed.weight": w.up_embed, "down_embed.weight": w.down_embed}, strict=False)
+    layer = layer.to(device).train()
+    bx, by = oracle.BNState.fresh(16), oracle.BNState.fresh(16)
+    g = torch.Generator().manual_seed(10)
+    for step in range(3):
+        x = torch.randn(1, T, H, generator=g) * (1.0 + step)
+        want, _, _ = oracle.moe_forward(x, w, bx, by, k, training=True, momentum=None)
+        got = layer(x.to(device))
+        assert layer.router_norm_x.num_batches_tracked.item() == step + 1 == int(bx.num_batches_tracked)
+        torch.testing.assert_close(layer.router_norm_x.running_mean.cpu(), bx.running_mean, rtol=1e-4, atol=1e-6)
+        torch.testing.assert_close(layer.router_norm_y.running_var.cpu(), by.running_var, rtol=1e-4, atol=1e-6)
+        torch.testing.assert_close(got.cpu(), want, rtol=1e-3, atol=1e-4)
+    layer.router_norm_y.momentum = 0.1
+    with pytest.raises(ValueError):                               # one momentum for both halves
+        layer(x.to(device))
+
+
 @pytest.mark.parametrize("training", [True, False], ids=["train", "eval"])
 @pytest.mark.parametrize("T", [1, 2, 3, 5, 31, 33, 65])
 def test_layer_tiny_token_counts(T, training, device):
@@ -418,6 +445,20 @@ def test_layer_tiny_token_counts(T, training, device):
     sd = {"gate_proj.weight": w.gate_proj, "up_proj.weight": w.up_proj, "down_proj.weight": w.down_proj,
           "router_gate_x.weight": w.router_gate_x, "router_gate_y.weight": w.router_gate_y,
           "up_embed.weight": w.up_embed, "down_embed.weight": w.down_embed}
+    if T == 1 and training:
+        # batch statistics of a single sample: nn.BatchNorm1d raises (reference omni_moe.py:70-71), and so do the oracle and the layer
+        with pytest.raises(ValueError):
+            oracle.moe_forward(x, w, oracle.BNState.fresh(16), oracle.BNState.fresh(16), k, training)
+        for overlap in (True, False):
+            layer = OmniMoE(OmniMoEConfig(H, I, "silu", N, k))
+            layer.load_state_dict(sd, strict=False)
+            layer = layer.to(device=device, dtype=torch.bfloat16).train()
+            layer.overlap_branches = overlap
+            layer.overlap_min_work = 0
+            with pytest.raises(ValueError, match="more than 1 value per channel"):
+                layer(x.to(device))
+            assert layer.router_norm_x.num_batches_tracked.item() == 0
+        return
     want, _, _ = oracle.moe_forward(x, w, oracle.BNState.fresh(16), oracle.BNState.fresh(16), k, training)
     outs = []
     for overlap in (True, False):

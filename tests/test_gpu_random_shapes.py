@@ -106,7 +106,7 @@ def test_layer_random_shapes_fp32(device):
         r = int(N ** 0.5)
         k = 2 * rng.randint(1, max(1, min(8, r * r // 2)))
         T = rng.choice([1, 5, 64, 200, 777])
-        training = rng.random() < 0.5
+        training = rng.random() < 0.5 and T > 1         # batch statistics of one sample raise, as nn.BatchNorm1d does
         x, w = oracle.make_layer_inputs(100 + case, T, H, I, N, dtype=torch.float32, w_std=0.1)
         sd = {"gate_proj.weight": w.gate_proj, "up_proj.weight": w.up_proj, "down_proj.weight": w.down_proj,
               "router_gate_x.weight": w.router_gate_x, "router_gate_y.weight": w.router_gate_y,

@@ -40,6 +40,29 @@ def test_batch_norm_matches_torch_module(dtype, training):
         torch.testing.assert_close(n.var(0, unbiased=False), torch.ones(r), rtol=1e-3, atol=1e-3)
 
 
+def test_batch_norm_cumulative_average_and_single_sample():
+    """momentum=None: the module averages the batch statistics cumulatively (factor 1 / num_batches_tracked); a single
+    sample in training raises, as nn.BatchNorm1d does."""
+    g = torch.Generator().manual_seed(3)
+    r = 24
+    bn = nn.BatchNorm1d(r, affine=False, momentum=None).train()
+    st = oracle.BNState.fresh(r)
+    for step in range(4):
+        z = torch.randn(50 + step, r, generator=g) * (1 + step) + step
+        want = bn(z)
+        got = oracle.batch_norm(z, st.running_mean, st.running_var, True, momentum=None, num_batches_tracked=st.num_batches_tracked)
+        st.num_batches_tracked += 1
+        torch.testing.assert_close(got, want, rtol=1e-5, atol=1e-5)
+        torch.testing.assert_close(st.running_mean, bn.running_mean, rtol=1e-5, atol=1e-6)
+        torch.testing.assert_close(st.running_var, bn.running_var, rtol=1e-5, atol=1e-6)
+    assert int(st.num_batches_tracked) == int(bn.num_batches_tracked) == 4
+    with pytest.raises(ValueError):
+        oracle.batch_norm(torch.randn(1, r), st.running_mean, st.running_var, True)
+    with pytest.raises(ValueError):
+        bn(torch.randn(1, r))
+    oracle.batch_norm(torch.randn(1, r), st.running_mean, st.running_var, False)      # eval takes one sample
+
+
 def test_batch_norm_bf16_matches_functional():
     g = torch.Generator().manual_seed(1)
     z = torch.randn(512, 64, generator=g).bfloat16()
