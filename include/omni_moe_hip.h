@@ -57,6 +57,14 @@ extern "C" {
 OMNI_API int32_t omni_abi_version(void);
 OMNI_API const char* omni_error_string(int32_t code);
 
+/* Optional one-time set-up of the CURRENT device: raises the dynamic-LDS limit of every kernel that needs more
+ * than the 64 KiB default and resolves the device scratch of omni_schedule_noalloc.  Every entry point does its
+ * share of this on first use, so calling omni_init() is only needed by callers that must not meet a
+ * non-stream HIP call later -- e.g. before the first HIP-graph capture of a shape that has not run eagerly.
+ * Needs a GPU; idempotent; call once per device, with that device current.  No counterpart in the reference
+ * (Triton compiles and configures its kernels on first launch). */
+OMNI_API int32_t omni_init(void);
+
 /* Cartesian-product router selection.
  * Replaces triton_omni_router_func / _omni_router_forward
  * (omni_moe/ops/triton/interface.py:32-51, omni_router.py:167-232, kernel :8-95)

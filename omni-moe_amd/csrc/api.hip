@@ -1,7 +1,14 @@
 // ABI bookkeeping of libomni_moe_hip.so: version and error strings.
 #include "omni_moe_hip.h"
+#include "common.h"
 
 extern "C" OMNI_API int32_t omni_abi_version(void) { return OMNI_ABI_VERSION; }
+
+extern "C" OMNI_API int32_t omni_init(void) {
+  for (omni::LdsKernel* k = omni::lds_kernel_list(); k; k = k->next)
+    if (hipError_t e = k->ensure(); e != hipSuccess) return OMNI_ERR_HIP_BASE + (int)e;
+  return omni::schedule_scratch_prepare();
+}
 
 extern "C" OMNI_API const char* omni_error_string(int32_t code) {
   switch (code) {

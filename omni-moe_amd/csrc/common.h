@@ -107,17 +107,36 @@ __device__ __forceinline__ float silu_fast(float x) {
 }
 
 // ---- host side ---------------------------------------------------------------
-// Raises a kernel's dynamic-LDS limit, once per device (the attribute belongs to the device's
-// copy of the kernel).  `done` is that kernel's bit mask of devices already set up; concurrent
-// callers at worst set the attribute twice.
-inline hipError_t ensure_dynamic_lds(const void* kernel, int bytes, std::atomic<uint64_t>& done) {
-  int dev = 0;
-  if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
-  const uint64_t bit = 1ull << (dev & 63);
-  if (done.load(std::memory_order_acquire) & bit) return hipSuccess;
-  if (hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes); e != hipSuccess) return e;
-  done.fetch_or(bit, std::memory_order_release);
-  return hipSuccess;
+// A kernel whose dynamic LDS exceeds the 64 KiB default needs its limit raised once per device (the
+// attribute belongs to the device's copy of the kernel).  Every such kernel is one LdsKernel object with
+// static storage: its constructor links it into a list at library load, so that omni_init() can raise all
+// limits up front (a caller that captures HIP graphs wants no hipFuncSetAttribute inside a capture), and
+// ensure() does it on first use for callers that never call omni_init().  `done` is the bit mask of devices
+// already set up; concurrent callers at worst set the attribute twice.
+struct LdsKernel;
+inline LdsKernel*& lds_kernel_list() {
+  static LdsKernel* head = nullptr;
+  return head;
 }
+struct LdsKernel {
+  const void* kernel;
+  int bytes;
+  std::atomic<uint64_t> done{0};
+  LdsKernel* next;
+  LdsKernel(const void* k, int b) : kernel(k), bytes(b), next(lds_kernel_list()) { lds_kernel_list() = this; }
+  hipError_t ensure() {
+    int dev = 0;
+    if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
+    const uint64_t bit = 1ull << (dev & 63);
+    if (done.load(std::memory_order_acquire) & bit) return hipSuccess;
+    if (hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes); e != hipSuccess) return e;
+    done.fetch_or(bit, std::memory_order_release);
+    return hipSuccess;
+  }
+};
+
+// The schedule's allocation-free entry point keeps a device array; this resolves its address on the
+// current device (defined beside the array).
+int schedule_scratch_prepare();
 
 }  // namespace omni

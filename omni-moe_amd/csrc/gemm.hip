@@ -611,6 +611,17 @@ __global__ __launch_bounds__(kGemmThreads, 1) void gemm_nt_dma_kernel(const Gemm
   OMNI_STAMP(3);
 }
 
+// One list entry per kernel instantiation that launch_gemm can start (the static members come into being
+// at library load for every instantiation the dispatch below names).
+template <int DT, int TM, int TN, int EPI, int BK, int NS>
+struct DmaKernelLds {
+  static inline LdsKernel entry{(const void*)gemm_nt_dma_kernel<DT, TM, TN, EPI, BK, NS>, NS * (2 * TM * 32 + 2 * TN * 32) * BK * 2};
+};
+template <int DT, int TM, int TN, int EPI>
+struct StagedKernelLds {
+  static inline LdsKernel entry{(const void*)gemm_nt_kernel<DT, TM, TN, EPI>, 2 * (2 * TM * 32 + 2 * TN * 32) * kRowBytes};
+};
+
 template <int DT, int TM, int TN, int EPI>
 static hipError_t launch_gemm(GemmArgs g, hipStream_t s) {
   constexpr int BM = 2 * TM * 32, BR = 2 * TN * 32, BN = (EPI == kEpiSwiglu) ? BR / 2 : BR;
@@ -635,14 +646,13 @@ static hipError_t launch_gemm(GemmArgs g, hipStream_t s) {
     constexpr int kDmaLds = kDmaStages * (BM + BR) * kDmaBK * 2;
     static_assert(kDmaLds <= 160 * 1024, "LDS ring exceeds 160 KiB");
     auto kern = gemm_nt_dma_kernel<DT, TM, TN, EPI, kDmaBK, kDmaStages>;
-    static std::atomic<uint64_t> configured{0};      // one per kernel instantiation
-    if (hipError_t e = ensure_dynamic_lds((const void*)kern, kDmaLds, configured); e != hipSuccess) return e;
+    static_assert(kDmaLds == kDmaStages * (2 * TM * 32 + 2 * TN * 32) * kDmaBK * 2, "list entry and launch disagree");
+    if (hipError_t e = DmaKernelLds<DT, TM, TN, EPI, kDmaBK, kDmaStages>::entry.ensure(); e != hipSuccess) return e;
     hipLaunchKernelGGL(kern, dim3(blocks), dim3(kGemmThreads), kDmaLds, s, g);
     return hipGetLastError();
   }
   auto kern = gemm_nt_kernel<DT, TM, TN, EPI>;       // any K % 8 == 0: staged through registers
-  static std::atomic<uint64_t> configured{0};
-  if (hipError_t e = ensure_dynamic_lds((const void*)kern, kLds, configured); e != hipSuccess) return e;
+  if (hipError_t e = StagedKernelLds<DT, TM, TN, EPI>::entry.ensure(); e != hipSuccess) return e;
   hipLaunchKernelGGL(kern, dim3(blocks), dim3(kGemmThreads), kLds, s, g);
   return hipGetLastError();
 }

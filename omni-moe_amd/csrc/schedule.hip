@@ -261,6 +261,9 @@ static bool make_plan(int64_t P, int64_t N, SortPlan* pl) {
   return true;
 }
 
+// up to 9 x 4104 counters exceed the 64 KiB default
+static LdsKernel g_scatter_lds{(const void*)sort_scatter_kernel, kMaxStride * (kSortWaves + 1) * 4};
+
 }  // namespace omni
 
 // workspace: hist [blocks][stride] | two-pass sorts only: keys A [P] | keys B [P] | pair ids [P]
@@ -289,9 +292,7 @@ extern "C" OMNI_API int32_t omni_schedule(const int32_t* indices, int32_t* offse
   int32_t* keys_b = (int32_t*)w;     w += align_up((size_t)P * 4 + 4, 256);
   int32_t* vals_a = (int32_t*)w;
 
-  static std::atomic<uint64_t> configured{0};              // tables of up to 8 x 4104 counters exceed the 64 KiB default
-  if (hipError_t e = ensure_dynamic_lds((const void*)sort_scatter_kernel, kMaxStride * (kSortWaves + 1) * 4, configured); e != hipSuccess)
-    return OMNI_ERR_HIP_BASE + (int)e;
+  if (hipError_t e = g_scatter_lds.ensure(); e != hipSuccess) return OMNI_ERR_HIP_BASE + (int)e;
   const bool single = pl.passes == 1;
   if (single || P > 0) {
     for (int pass = 0; pass < pl.passes; ++pass) {
@@ -354,6 +355,11 @@ static int scratch_address(void** out) {
   }
   *out = p;
   return OMNI_OK;
+}
+
+int schedule_scratch_prepare() {
+  void* p = nullptr;
+  return scratch_address(&p);
 }
 
 }  // namespace omni

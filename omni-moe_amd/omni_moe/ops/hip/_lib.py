@@ -26,6 +26,7 @@ DTYPE_CODE = {torch.bfloat16: OMNI_BF16, torch.float16: OMNI_F16, torch.float32:
 SIGNATURES = {
     "omni_abi_version": (c_int32, []),
     "omni_error_string": (c_char_p, [c_int32]),
+    "omni_init": (c_int32, []),
     "omni_router_select": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int32, c_int32, c_int32, c_void_p]),
     "omni_schedule_workspace_bytes": (c_size_t, [c_int64, c_int32, c_int64]),
     "omni_schedule": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int32, c_int64, c_void_p, c_void_p]),
@@ -89,6 +90,9 @@ def check(code: int, what: str) -> None:
     raise OmniHipError(f"{what}: {msg} (code {code})")
 
 
+_prepared_devices = set()
+
+
 def require_gpu(*tensors: torch.Tensor) -> torch.device:
     dev = tensors[0].device
     if dev.type != "cuda":
@@ -96,6 +100,12 @@ def require_gpu(*tensors: torch.Tensor) -> torch.device:
     for t in tensors:
         if t.device != dev:
             raise ValueError("all tensors must be on the same device")
+    if dev.index not in _prepared_devices:
+        # kernel attributes and the device scratch, once per device and before any launch, so that none of it
+        # can fall inside a later stream capture
+        with torch.cuda.device(dev):
+            check(load().omni_init(), "omni_init")
+        _prepared_devices.add(dev.index)
     return dev
 
 

@@ -320,8 +320,9 @@ class OmniLinearFunc(torch.autograd.Function):
 
 def hip_swiglu_func(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
     """silu(gate) * up element-wise, fp32 inside, one rounding (``TritonSwiGLUFunc``, reference omni_mlp.py:359-371)."""
-    if gate.shape != up.shape or gate.dtype != up.dtype or gate.dtype not in _lib.DTYPE_CODE:
-        raise ValueError("gate and up must match in shape and dtype (bfloat16, float16 or float32)")
+    assert gate.shape == up.shape, "gate and up must have the same shape"       # the reference asserts (utils.py:68-78)
+    if gate.dtype != up.dtype or gate.dtype not in _lib.DTYPE_CODE:
+        raise ValueError("gate and up must share one dtype (bfloat16, float16 or float32)")
     _lib.require_gpu(gate, up)
     if _needs_grad(gate, up):
         return OmniSwiGLUFunc.apply(gate, up)
@@ -340,8 +341,9 @@ def _swiglu_forward(gate, up):
 
 def hip_swiglu_bwd_func(dout, gate, up):
     """(dgate, dup) of ``hip_swiglu_func`` (reference omni_mlp.py:306-356)."""
-    if dout.shape != gate.shape or gate.shape != up.shape or len({dout.dtype, gate.dtype, up.dtype}) != 1:
-        raise ValueError("dout, gate and up must match in shape and dtype")
+    assert dout.shape == gate.shape == up.shape, "dout, gate and up must have the same shape"
+    if len({dout.dtype, gate.dtype, up.dtype}) != 1:
+        raise ValueError("dout, gate and up must share one dtype")
     _lib.require_gpu(dout, gate, up)
     dout, gate, up = _c(dout), _c(gate), _c(up)
     dgate, dup = torch.empty_like(gate), torch.empty_like(up)

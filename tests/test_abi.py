@@ -82,6 +82,13 @@ def test_argument_errors_need_no_gpu():
     assert moe(64, 64, 16, 4, 2, dt=5) == -3
     assert lib.omni_mlp_fwd(p, p, p, p, None, p, 4, 64, 64, 0, None, None) == -6 # no workspace
     assert lib.omni_schedule_workspace_bytes(4, 2, 100) >= 200
+    # batch statistics of a single token: nn.BatchNorm1d raises in training (reference omni_moe.py:70-71), the library refuses
+    assert lib.omni_moe_fwd(*([p] * 15), 1, 64, 64, 16, 4, 2, 0, 2, 1, 0.1, 1e-5, p, None, None, None, None) == -2
+    assert lib.omni_router_fwd(*([p] * 9), 1, 0.1, 1e-5, p, p, None, 1, 64, 4, 2, 0, 2, p, None) == -2
+    assert lib.omni_router_fwd(p, p, p, p, p, None, p, p, None, 1, -1.0, 1e-5, p, p, None, 4, 64, 4, 2, 0, 2, p, None) == -1   # cumulative average needs the counters
+    import torch
+    if not torch.cuda.is_available():
+        assert lib.omni_init() >= 1000           # a HIP error (no device), not a crash
 
 
 def test_ops_fail_loudly_without_gpu():

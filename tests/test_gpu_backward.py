@@ -163,8 +163,10 @@ def test_swiglu_fwd_bwd(dtype, device):
     da, db = hip.hip_swiglu_bwd_func(d.to(device), a.to(device), b.to(device))
     _close(da, ca.grad, dtype, "dgate")
     _close(db, cb.grad, dtype, "dup")
-    with pytest.raises(ValueError):
+    with pytest.raises(AssertionError):                       # as the reference's assert_omni_mlp_fwd_inputs (utils.py:68-78)
         hip.hip_swiglu_func(a.to(device), b.to(device)[:, :8])
+    with pytest.raises(ValueError):
+        hip.hip_swiglu_func(a.to(device), b.to(device).to(torch.float16 if dtype != torch.float16 else torch.float32))
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
