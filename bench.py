@@ -306,6 +306,23 @@ def main():
         m, b = time_launches(torch, lambda: hip.hip_omni_expert_func(x3, up3, down3, g3, i3, algo="segment"))
         kernels.append(hbm_entry("expert op, expert-centric 'segment' algorithm (schedule + scores pass + token pass), c3", m, b,
                                  expert_alg_bytes(T3, H, k), note="for comparison; same results as the gather algorithm"))
+        # the reference's group regime (omni_scheduler.py:58: tokens x k / experts > 256): same tokens, 256 experts; AUTO takes
+        # the dense algorithm (two MFMA GEMMs over all experts), timed beside the gather algorithm on the same inputs
+        Ng = 256
+        xg_c, upg_c, downg_c, gg_c, ig_c = oracle.make_expert_inputs(2, T3, H, Ng, k)
+        xg, upg, downg, gg, ig = (t.to(dev) for t in (xg_c, upg_c, downg_c, gg_c, ig_c))
+        yg = hip.hip_omni_expert_func(xg, upg, downg, gg, ig, algo="dense")
+        wantg = oracle.expert_forward(xg_c[:sub], upg_c, downg_c, gg_c[:sub], ig_c[:sub])
+        torch.testing.assert_close(yg[:sub].float().cpu(), wantg.float(), rtol=2e-2, atol=2e-2)
+        m, b = time_launches(torch, lambda: hip.hip_omni_expert_func(xg, upg, downg, gg, ig))
+        dense = mfma_entry("expert op, dense algorithm (gate rows + transpose + two MFMA GEMMs), group regime: 16384 tokens, 256 experts, top-16",
+                           2 * T3 * H * Ng + 2 * T3 * H * 2 * Ng, m, b, None, None)
+        m, b = time_launches(torch, lambda: hip.hip_omni_expert_func(xg, upg, downg, gg, ig, algo="gather"))
+        dense["gather_algorithm_ms"] = m
+        dense["note"] = ("1024 pairs per expert: every token meets every expert in a [T,N] product; the flop count is the dense one "
+                         "(6 T H N), the selected pairs alone would be 4 T k H")
+        kernels.append(dense)
+        del xg, upg, downg, gg, ig, yg
         if "train" in sections:
             # training path (not part of the forward metric): backward of the expert op at the same shape
             dy3 = x3 * 0.5
