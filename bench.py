@@ -41,7 +41,8 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 # Bytes that cross the fabric per launch (FETCH_SIZE + WRITE_SIZE of rocprofv3 --pmc, each scaled by a plain copy of
 # known size); counters cannot be read in-process, so these are the figures of the committed summaries named here.
 TRAFFIC_SOURCE = "profiles/bench_layer_c4_hbm_counters.txt, profiles/expert_c5_hbm_counters.txt"
-TRAFFIC_BYTES = {"expert_c3": 183.2e6, "expert_c4": 57.8e6, "expert_gather_c3": 897.9e6, "gateup_c4": 134.7e6, "down_c4": 117.6e6,
+TRAFFIC_BYTES = {"expert_c3": 182.8e6, "expert_c4": 57.8e6, "expert_gather_c3": 898.5e6, "gateup_c4": 134.7e6, "down_c4": 117.6e6,
+                 "down_plain_c4": 109.2e6, "schedule_c3": 13.34e6,
                  "expert_c5_routed": 1029.2e6, "expert_c5_uniform": 8846.8e6}
 SECTIONS = ("layer", "kernels", "expert_c3", "expert_c5", "probe", "train", "cpu")
 
@@ -268,7 +269,7 @@ def main():
         m, b = time_launches(torch, lambda: hip.hip_linear_func(h, layer.down_proj.weight, e_out))
         kernels.append(mfma_entry("gemm_nt_dma_kernel<residual> (down projection + experts add), c4", 2 * T * H * I, m, b, TRAFFIC_BYTES["down_c4"], sustained))
         m, b = time_launches(torch, lambda: hip.hip_linear_func(h, layer.down_proj.weight))
-        kernels.append(mfma_entry("gemm_nt_dma_kernel<plain> (down projection alone, as on the two-stream path), c4", 2 * T * H * I, m, b, None, sustained))
+        kernels.append(mfma_entry("gemm_nt_dma_kernel<plain> (down projection alone, as on the two-stream path), c4", 2 * T * H * I, m, b, TRAFFIC_BYTES["down_plain_c4"], sustained))
         m, b = time_launches(torch, lambda: hip.hip_add_inplace_func(y0, e_out))
         kernels.append(hbm_entry("add_inplace_kernel (join of the two branches), c4", m, b, 3 * T * H * 2, resident_in_hbm=False,
                                  note="24 MiB that the caches hold between launches"))
@@ -302,7 +303,9 @@ def main():
                                  TRAFFIC_BYTES["expert_gather_c3"], expert_min_bytes(T3, H, N, k),
                                  note="for comparison: whole rows per wave, three quarters of them fetched over the fabric"))
         m, b = time_launches(torch, lambda: hip.hip_omni_schedule_func(i3, N))
-        kernels.append(hbm_entry("schedule (stable counting sort of the pairs by expert), c3", m, b, T3 * k * 14 + 8 * (N + 1)))
+        kernels.append(hbm_entry("schedule (stable counting sort of the pairs by expert: sort_count_kernel + sort_scatter_kernel), c3", m, b,
+                                 T3 * k * 12 + 4 * (N + 1), TRAFFIC_BYTES["schedule_c3"],
+                                 note="ids in, pair ids + token ids + offsets out; bounded by per-block work on the 4097-bin tables, not by bytes"))
         m, b = time_launches(torch, lambda: hip.hip_omni_expert_func(x3, up3, down3, g3, i3, algo="segment"))
         kernels.append(hbm_entry("expert op, expert-centric 'segment' algorithm (schedule + scores pass + token pass), c3", m, b,
                                  expert_alg_bytes(T3, H, k), note="for comparison; same results as the gather algorithm"))
