@@ -9,15 +9,17 @@
 //            them as one row of hist[block][bin] (coalesced, 16-bit counters: a tile has fewer
 //            than 65536 pairs; the histogram is the only scratch);
 //   scatter: every block sums the rows of hist (all of them for the bins' totals, the rows above
-//            its own for its share), scans the totals over the bins, and has its output bases;
-//            block 0 writes them out as the segment offsets.  Then it places its tile.
+//            its own tile for its share), scans the totals over the bins, and has its output
+//            bases; block 0 writes them out as the segment offsets.  Then it places its pairs.
+// Scattered 4-byte stores are bound by the requests one CU can issue, so up to 8 scatter blocks share
+// a tile: each places one part of it and counts the parts before its own itself.
 // The scatter is order preserving without any global atomic: each of the block's 8 waves owns a
-// contiguous eighth of the tile; per-wave bin bases come from an LDS table, and inside a wave 64
-// consecutive items rank themselves with ballots.  So a segment lists its pairs by ascending pair
-// id, and the result is bit-identical from run to run.  Offsets are dense over all N experts (an
-// unused expert has an empty segment), so no compaction pass is needed, and nothing returns to
-// the host.  Few, large tiles (about 131072 / bins blocks) keep the histogram small: it is read
-// once per block.
+// contiguous eighth of the part; per-wave bin bases come from an LDS table, and inside a wave 64
+// consecutive items rank themselves (an LDS add per item, ballots where two items of a step meet
+// in a bin).  So a segment lists its pairs by ascending pair id, and the result is bit-identical
+// from run to run.  Offsets are dense over all N experts (an unused expert has an empty segment),
+// so no compaction pass is needed, and nothing returns to the host.  Few, large tiles (32 where the
+// 16-bit counters allow) keep the histogram small: every scatter block reads it once, one batch of loads.
 #include "common.h"
 #include "omni_moe_hip.h"
 
@@ -30,7 +32,7 @@ constexpr int kBinChunk = 8;                              // bins a thread sums 
 constexpr int kMaxStride = (kMaxBins + kBinChunk - 1) / kBinChunk * kBinChunk;
 constexpr int kMaxSortBlocks = 1024;
 constexpr int kMaxTile = 63 * 1024;                       // counters are 16 bits wide
-constexpr int kRowBatch = 16;                             // histogram rows whose loads are in flight together
+constexpr int kRowBatch = 32;                             // histogram rows whose loads are in flight together
 static_assert(kMaxBins <= kSortThreads * kBinChunk + 1, "the scan covers 8 bins per thread plus one");
 
 struct SortPass {
@@ -44,6 +46,7 @@ struct SortPass {
   int64_t num_pairs;
   int tile;                 // pairs per block, a multiple of 1024
   int blocks, bins, stride, bits;   // stride = bins rounded up to 8; bits = ceil(log2(bins))
+  int sub;                  // scatter blocks per tile (a power of two that divides tile / 8)
   int shift;                // digit = id >> shift ...
   uint32_t mask;            //   ... & mask (0xFFFFFFFF on the last pass)
   int last;                 // last pass: ids outside [0, N) go to bin bins-1; earlier passes: to bin 0
@@ -63,7 +66,18 @@ __global__ __launch_bounds__(kSortThreads) void sort_count_kernel(const SortPass
   __syncthreads();
   const int64_t t0 = (int64_t)blockIdx.x * a.tile;
   const int64_t t1 = t0 + a.tile < a.num_pairs ? t0 + a.tile : a.num_pairs;
-  for (int64_t i = t0 + threadIdx.x; i < t1; i += kSortThreads) atomicAdd(&cnt[sort_digit(a, a.keys_in[i])], 1);
+  constexpr int kBatch = 8;                              // loads in flight per thread
+  for (int64_t i0 = t0 + threadIdx.x; i0 < t1; i0 += kBatch * kSortThreads) {
+    int32_t key[kBatch];
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) {
+      const int64_t i = i0 + u * kSortThreads;
+      key[u] = i < t1 ? a.keys_in[i] : 0;
+    }
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u)
+      if (i0 + u * kSortThreads < t1) atomicAdd(&cnt[sort_digit(a, key[u])], 1);
+  }
   __syncthreads();
   for (int d = threadIdx.x; d < a.stride; d += kSortThreads) a.hist[(int64_t)blockIdx.x * a.stride + d] = (uint16_t)cnt[d];
 }
@@ -73,52 +87,89 @@ __global__ __launch_bounds__(kSortThreads) void sort_scatter_kernel(const SortPa
   __shared__ int32_t wave_tot[kSortWaves];
   int32_t* bin_base = tbl + kSortWaves * a.stride;
   const int lane = lane_id(), wave = threadIdx.x >> 6;
-  for (int d = threadIdx.x * 4; d < a.stride * kSortWaves; d += kSortThreads * 4) *(u32x4_t*)(tbl + d) = u32x4_t{0, 0, 0, 0};   // stride % 8 == 0
-  __syncthreads();
-  const int64_t t0 = (int64_t)blockIdx.x * a.tile;
-  const int64_t t1 = t0 + a.tile < a.num_pairs ? t0 + a.tile : a.num_pairs;
-  const int per_wave = a.tile / kSortWaves;
-  const int64_t w0 = t0 + (int64_t)wave * per_wave < t1 ? t0 + (int64_t)wave * per_wave : t1;   // this wave's eighth, in order
-  const int64_t w1 = w0 + per_wave < t1 ? w0 + per_wave : t1;
-  int32_t* mine = tbl + wave * a.stride;
-  for (int64_t i = w0 + lane; i < w1; i += kWave) atomicAdd(&mine[sort_digit(a, a.keys_in[i])], 1);
-  __syncthreads();
-
-  // Output bases.  Thread t takes bins 8t .. 8t+7 and walks down the histogram rows: the rows above this block's
-  // give what earlier tiles put into each bin, all rows the bin's total.  An exclusive scan of the totals over the
-  // bins (thread order = bin order) gives each bin's first position.  The rows come from other blocks' writes, i.e.
-  // from memory: the loads of kRowBatch rows are in flight together.  512 threads cover 4096 bins; the one bin
-  // beyond them (ids outside the table, when there are 4096 experts) is summed by wave 0, a row per lane.
+  // The histogram rows come from other blocks' writes, i.e. from memory: thread t takes bins 8t .. 8t+7 of every row
+  // (one 16-byte load per row), kRowBatch rows in flight together, the first batch while the tile is being counted.
   const int d0 = threadIdx.x * kBinChunk;
   const bool active = d0 < a.stride && d0 < kSortThreads * kBinChunk;
+  auto load_rows = [&](u32x4_t (&row)[kRowBatch], int first) {
+#pragma unroll
+    for (int j = 0; j < kRowBatch; ++j)
+      row[j] = (active && first + j < a.blocks) ? *(const u32x4_t*)(a.hist + (int64_t)(first + j) * a.stride + d0) : u32x4_t{0, 0, 0, 0};
+  };
+  u32x4_t early[kRowBatch];
+  load_rows(early, 0);
+  for (int d = threadIdx.x * 4; d < a.stride * (kSortWaves + 1); d += kSortThreads * 4) *(u32x4_t*)(tbl + d) = u32x4_t{0, 0, 0, 0};   // stride % 8 == 0
+  __syncthreads();
+  // a.sub blocks share a tile (the scattered stores are bound by the requests one CU can issue, so they are spread
+  // over many CUs); block sb of a tile places the sb-th part of it, after the parts before it
+  const int tile_idx = (int)blockIdx.x / a.sub, sb = (int)blockIdx.x % a.sub;
+  const int64_t t0 = (int64_t)tile_idx * a.tile;
+  const int64_t t1 = t0 + a.tile < a.num_pairs ? t0 + a.tile : a.num_pairs;
+  const int share = a.tile / a.sub, per_wave = share / kSortWaves;
+  const int64_t s0 = t0 + (int64_t)sb * share < t1 ? t0 + (int64_t)sb * share : t1;             // earlier parts of the tile: [t0, s0)
+  const int64_t w0 = s0 + (int64_t)wave * per_wave < t1 ? s0 + (int64_t)wave * per_wave : t1;   // this wave's eighth of the part, in order
+  const int64_t w1 = w0 + per_wave < t1 ? w0 + per_wave : t1;
+  int32_t* mine = tbl + wave * a.stride;
+  constexpr int kGroup = 8;                              // steps of 64 items whose loads are issued together
+  for (int64_t i0 = t0 + threadIdx.x; i0 < s0; i0 += kGroup * kSortThreads) {   // what the tile's earlier parts put into each bin
+    int32_t key[kGroup];
+#pragma unroll
+    for (int u = 0; u < kGroup; ++u) {
+      const int64_t i = i0 + u * kSortThreads;
+      key[u] = i < s0 ? a.keys_in[i] : 0;
+    }
+#pragma unroll
+    for (int u = 0; u < kGroup; ++u)
+      if (i0 + u * kSortThreads < s0) atomicAdd(&bin_base[sort_digit(a, key[u])], 1);
+  }
+  for (int64_t g0 = w0; g0 < w1; g0 += kGroup * kWave) {
+    int32_t key[kGroup];
+#pragma unroll
+    for (int u = 0; u < kGroup; ++u) {
+      const int64_t i = g0 + u * kWave + lane;
+      key[u] = i < w1 ? a.keys_in[i] : 0;
+    }
+#pragma unroll
+    for (int u = 0; u < kGroup; ++u)
+      if (g0 + u * kWave + lane < w1) atomicAdd(&mine[sort_digit(a, key[u])], 1);
+  }
+  __syncthreads();
+
+  // Output bases.  The rows above this block's give what earlier tiles put into each bin, all rows the bin's total.
+  // An exclusive scan of the totals over the bins (thread order = bin order) gives each bin's first position.
+  // 512 threads cover 4096 bins; the one bin beyond them (ids outside the table, when there are 4096 experts) is
+  // summed by wave 0, a row per lane.
   int32_t before[kBinChunk], rest[kBinChunk];
 #pragma unroll
   for (int i = 0; i < kBinChunk; ++i) before[i] = rest[i] = 0;
-  auto add_rows = [&](int32_t (&acc)[kBinChunk], int first, int end) {
-    for (int b0 = first; b0 < end; b0 += kRowBatch) {
-      u32x4_t row[kRowBatch];
+  auto add_rows = [&](const u32x4_t (&row)[kRowBatch], int first) {
 #pragma unroll
-      for (int j = 0; j < kRowBatch; ++j)
-        row[j] = (active && b0 + j < end) ? *(const u32x4_t*)(a.hist + (int64_t)(b0 + j) * a.stride + d0) : u32x4_t{0, 0, 0, 0};
+    for (int j = 0; j < kRowBatch; ++j) {
+      const bool above = first + j < tile_idx;            // uniform
 #pragma unroll
-      for (int j = 0; j < kRowBatch; ++j)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const uint32_t pair = row[j][i];
-          acc[2 * i] += (int32_t)(pair & 0xffffu);
-          acc[2 * i + 1] += (int32_t)(pair >> 16);
-        }
+      for (int i = 0; i < 4; ++i) {
+        const uint32_t pair = row[j][i];
+        const int32_t lo = (int32_t)(pair & 0xffffu), hi = (int32_t)(pair >> 16);
+        before[2 * i] += above ? lo : 0;
+        before[2 * i + 1] += above ? hi : 0;
+        rest[2 * i] += above ? 0 : lo;
+        rest[2 * i + 1] += above ? 0 : hi;
+      }
     }
   };
-  add_rows(before, 0, (int)blockIdx.x);
-  add_rows(rest, (int)blockIdx.x, a.blocks);
+  add_rows(early, 0);
+  for (int b0 = kRowBatch; b0 < a.blocks; b0 += kRowBatch) {
+    u32x4_t row[kRowBatch];
+    load_rows(row, b0);
+    add_rows(row, b0);
+  }
   const int tail_bin = kSortThreads * kBinChunk;         // 4096
   int32_t tail_before = 0, tail_total = 0;
   if (a.bins > tail_bin && wave == 0) {
     for (int b = lane; b < a.blocks; b += kWave) {
       const int32_t c = a.hist[(int64_t)b * a.stride + tail_bin];
       tail_total += c;
-      tail_before += b < (int)blockIdx.x ? c : 0;
+      tail_before += b < tile_idx ? c : 0;
     }
 #pragma unroll
     for (int m = kWave / 2; m >= 1; m >>= 1) {
@@ -149,13 +200,13 @@ __global__ __launch_bounds__(kSortThreads) void sort_scatter_kernel(const SortPa
       const int d = d0 + i;
       if (active && d < a.bins) {
         if (a.offsets_out && blockIdx.x == 0) a.offsets_out[d] = excl;
-        bin_base[d] = excl + before[i];
+        bin_base[d] += excl + before[i];                   // on top of the earlier parts' count
       }
       excl += before[i] + rest[i];
     }
     if (a.bins > tail_bin && threadIdx.x == 0) {         // the bin behind all others starts where they end
       if (a.offsets_out && blockIdx.x == 0) a.offsets_out[tail_bin] = all;
-      bin_base[tail_bin] = all + tail_before;
+      bin_base[tail_bin] += all + tail_before;
     }
     __syncthreads();
   }
@@ -171,10 +222,14 @@ __global__ __launch_bounds__(kSortThreads) void sort_scatter_kernel(const SortPa
   }
   __syncthreads();
 
+  // Placement, 64 consecutive items at a time and in order.  Position = the bin's running base + the number of earlier
+  // lanes of the step with the same bin.  Every lane reads the base, then bumps it; a lane that finds the base already
+  // bumped shares its bin with another lane of its step, and only then are the lanes of that bin ranked by lane number
+  // (whatever order the adds took effect in).  LDS executes a wave's instructions in order, so the reads and adds of all
+  // steps of a group are issued back to back (a later step sees the earlier steps' adds) and waited for once.
   const uint64_t below = (1ull << lane) - 1ull;
-  constexpr int kGroup = 8;                                  // steps whose loads are issued together
   for (int64_t g0 = w0; g0 < w1; g0 += kGroup * kWave) {
-    int32_t keys[kGroup], vals[kGroup];
+    int32_t keys[kGroup], vals[kGroup], dig[kGroup], pos[kGroup], bumped[kGroup];
 #pragma unroll
     for (int u = 0; u < kGroup; ++u) {
       const int64_t i = g0 + u * kWave + lane;
@@ -182,31 +237,31 @@ __global__ __launch_bounds__(kSortThreads) void sort_scatter_kernel(const SortPa
       vals[u] = i < w1 ? (a.vals_in ? a.vals_in[i] : (int32_t)i) : 0;
     }
 #pragma unroll
-    for (int u = 0; u < kGroup; ++u) {                       // 64 consecutive items at a time, in order
-      const int64_t i = g0 + u * kWave + lane;
-      const bool active = i < w1;
-      const int32_t key = keys[u], val = vals[u];
-      const int d = active ? sort_digit(a, key) : 0;
-      // Position = the bin's running base + the number of earlier lanes of this step with the same bin.  Every lane
-      // reads the base, then bumps it; a lane that finds the base already bumped shares its bin with another lane of
-      // the step.  Only then are the lanes of that bin ranked by lane number (whatever order the adds took effect in).
-      int32_t pos = 0, bumped = 0;
+    for (int u = 0; u < kGroup; ++u) {
+      const bool active = g0 + u * kWave + lane < w1;
+      dig[u] = active ? sort_digit(a, keys[u]) : 0;
+      pos[u] = bumped[u] = 0;
       if (active) {
-        pos = mine[d];
-        bumped = atomicAdd(&mine[d], 1);
+        pos[u] = mine[dig[u]];
+        bumped[u] = atomicAdd(&mine[dig[u]], 1);
       }
-      uint64_t shared = __ballot(active && bumped != pos);   // the non-first lanes of shared bins
+    }
+#pragma unroll
+    for (int u = 0; u < kGroup; ++u) {
+      const bool active = g0 + u * kWave + lane < w1;
+      const int d = dig[u];
+      uint64_t shared = __ballot(active && bumped[u] != pos[u]);   // the non-first lanes of shared bins
       while (shared) {
         const int l = __builtin_ctzll(shared);
         const int v = __shfl(d, l, kWave);
-        const uint64_t grp = __ballot(active && d == v);     // all lanes of that bin; they read the same base
-        if (active && d == v) pos += __popcll(grp & below);
+        const uint64_t grp = __ballot(active && d == v);           // all lanes of that bin; they read the same base
+        if (active && d == v) pos[u] += __popcll(grp & below);
         shared &= ~grp;
       }
       if (active) {
-        if (a.keys_out) a.keys_out[pos] = key;
-        a.vals_out[pos] = val;
-        if (a.tok_out) a.tok_out[pos] = (int32_t)(((uint64_t)(uint32_t)val * a.inv_top_k) >> 40);   // val / top_k
+        if (a.keys_out) a.keys_out[pos[u]] = keys[u];
+        a.vals_out[pos[u]] = vals[u];
+        if (a.tok_out) a.tok_out[pos[u]] = (int32_t)(((uint64_t)(uint32_t)vals[u] * a.inv_top_k) >> 40);   // val / top_k
       }
     }
   }
@@ -231,7 +286,7 @@ static inline int ceil_log2(uint64_t v) { int b = 0; while ((1ull << b) < v) ++b
 
 // How the sort of P pairs with ids below N is split into passes and tiles.
 struct SortPlan {
-  int passes, lo_bits, bins[2], stride, tile, blocks;
+  int passes, lo_bits, bins[2], stride, tile, blocks, sub;
   size_t hist_entries;
 };
 static bool make_plan(int64_t P, int64_t N, SortPlan* pl) {
@@ -245,10 +300,9 @@ static bool make_plan(int64_t P, int64_t N, SortPlan* pl) {
   const int maxb = pl->bins[0] > pl->bins[1] ? pl->bins[0] : pl->bins[1];
   if (maxb > kMaxBins) return false;                       // N > 16 Mi experts
   pl->stride = (maxb + kBinChunk - 1) / kBinChunk * kBinChunk;
-  // every block reads the whole histogram: about 128 Ki counters of it (32 tiles at 4097 bins, 256 at 512),
-  // more where a tile would outgrow its 16-bit counters
-  int want = ((1 << 17) + maxb - 1) / maxb;
-  want = want < 1 ? 1 : (want > 256 ? 256 : want);
+  // every scatter block sums the whole histogram, one 16-byte load per row and thread: 32 rows (tiles) are one batch of
+  // loads; more only where a tile would outgrow its 16-bit counters
+  constexpr int want = 32;
   int64_t tile = (P + want - 1) / want;
   tile = (tile + 1023) / 1024 * 1024;
   if (tile < 1024) tile = 1024;
@@ -258,6 +312,9 @@ static bool make_plan(int64_t P, int64_t N, SortPlan* pl) {
   pl->blocks = (int)((P + tile - 1) / tile);
   if (pl->blocks < 1) pl->blocks = 1;
   pl->hist_entries = (size_t)pl->stride * pl->blocks;
+  // scatter blocks per tile: towards one block per CU, each part at least 8 waves x 64 items (tile is a multiple of 1024)
+  pl->sub = 1;
+  while (pl->sub < 8 && pl->blocks * pl->sub * 2 <= 256 && pl->tile / (pl->sub * 2) >= 512) pl->sub *= 2;
   return true;
 }
 
@@ -308,6 +365,7 @@ extern "C" OMNI_API int32_t omni_schedule(const int32_t* indices, int32_t* offse
       a.num_pairs = P;
       a.tile = pl.tile;
       a.blocks = pl.blocks;
+      a.sub = pl.sub;
       a.bins = pl.bins[pass];
       a.stride = pl.stride;
       a.bits = ceil_log2((uint64_t)a.bins);
@@ -317,7 +375,7 @@ extern "C" OMNI_API int32_t omni_schedule(const int32_t* indices, int32_t* offse
       a.num_experts = (uint32_t)N;
       a.inv_top_k = num_experts_per_token > 0 ? ((1ull << 40) + num_experts_per_token - 1) / (uint64_t)num_experts_per_token : 0;
       hipLaunchKernelGGL(sort_count_kernel, dim3(a.blocks), dim3(kSortThreads), (size_t)a.stride * 4, s, a);
-      hipLaunchKernelGGL(sort_scatter_kernel, dim3(a.blocks), dim3(kSortThreads), (size_t)a.stride * (kSortWaves + 1) * 4, s, a);
+      hipLaunchKernelGGL(sort_scatter_kernel, dim3(a.blocks * a.sub), dim3(kSortThreads), (size_t)a.stride * (kSortWaves + 1) * 4, s, a);
     }
   }
   if (!single) {
