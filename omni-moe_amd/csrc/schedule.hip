@@ -143,18 +143,17 @@ __global__ __launch_bounds__(kSortThreads) void sort_scatter_kernel(const SortPa
 #pragma unroll
   for (int i = 0; i < kBinChunk; ++i) before[i] = rest[i] = 0;
   auto add_rows = [&](const u32x4_t (&row)[kRowBatch], int first) {
-#pragma unroll
-    for (int j = 0; j < kRowBatch; ++j) {
-      const bool above = first + j < tile_idx;            // uniform
+    auto add = [&](int32_t (&acc)[kBinChunk], const u32x4_t& r) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const uint32_t pair = row[j][i];
-        const int32_t lo = (int32_t)(pair & 0xffffu), hi = (int32_t)(pair >> 16);
-        before[2 * i] += above ? lo : 0;
-        before[2 * i + 1] += above ? hi : 0;
-        rest[2 * i] += above ? 0 : lo;
-        rest[2 * i + 1] += above ? 0 : hi;
+        acc[2 * i] += (int32_t)(r[i] & 0xffffu);
+        acc[2 * i + 1] += (int32_t)(r[i] >> 16);
       }
+    };
+#pragma unroll
+    for (int j = 0; j < kRowBatch; ++j) {
+      if (first + j < tile_idx) add(before, row[j]);      // a scalar branch: the row index is uniform
+      else add(rest, row[j]);
     }
   };
   add_rows(early, 0);
