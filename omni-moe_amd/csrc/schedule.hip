@@ -6,20 +6,24 @@
 // N <= 4096 (one bin per expert), two passes (low then high half of the id bits) above that.
 // A pass is two kernels:
 //   count:   every block counts the bins of its contiguous tile of the input in LDS and writes
-//            them as one row of hist[block][bin] (coalesced, 16-bit counters: a tile has fewer
-//            than 65536 pairs; the histogram is the only scratch);
-//   scatter: every block sums the rows of hist (all of them for the bins' totals, the rows above
-//            its own tile for its share), scans the totals over the bins, and has its output
-//            bases; block 0 writes them out as the segment offsets.  Then it places its pairs.
-// Scattered 4-byte stores are bound by the requests one CU can issue, so up to 8 scatter blocks share
-// a tile: each places one part of it and counts the parts before its own itself.
+//            them as one row of hist[tile][bin] (16-bit counters: a tile has fewer than 65536
+//            pairs), plus the row's sum over each of the 8 bin slices;
+//   scatter: the bins are cut into 8 slices and a block places the pairs of ONE tile that fall
+//            into ONE slice.  It sums its slice of the hist rows (all rows for the bins' totals,
+//            the rows above its tile for its share), the slice sums of the slices below it, scans
+//            the totals, and has its output bases; the blocks of tile 0 write them out as the
+//            segment offsets.
+// Why slices: the scattered 4-byte stores are what the pass costs.  Slice s belongs to the blocks
+// with blockIdx % 8 == s, which the dispatcher places on XCD s, so every output line is written
+// through ONE L2 (which merges the stores of a line before it goes to memory) and the stores are
+// spread over all CUs; and a block's tables cover an eighth of the bins, so zeroing, summing,
+// scanning them is an eighth of the work.  The price is that a tile's keys are read by 8 blocks.
 // The scatter is order preserving without any global atomic: each of the block's 8 waves owns a
-// contiguous eighth of the part; per-wave bin bases come from an LDS table, and inside a wave 64
+// contiguous eighth of the tile; per-wave bin bases come from an LDS table, and inside a wave 64
 // consecutive items rank themselves (an LDS add per item, ballots where two items of a step meet
 // in a bin).  So a segment lists its pairs by ascending pair id, and the result is bit-identical
 // from run to run.  Offsets are dense over all N experts (an unused expert has an empty segment),
-// so no compaction pass is needed, and nothing returns to the host.  Few, large tiles (32 where the
-// 16-bit counters allow) keep the histogram small: every scatter block reads it once, one batch of loads.
+// so no compaction pass is needed, and nothing returns to the host.
 #include "common.h"
 #include "omni_moe_hip.h"
 
@@ -27,13 +31,15 @@ namespace omni {
 
 constexpr int kSortThreads = 512;
 constexpr int kSortWaves = kSortThreads / kWave;
+constexpr int kSlices = 8;                                // bin slices = XCDs
 constexpr int kMaxBins = 4097;                            // 4096 experts (or id slices) + 1 bin for ids outside [0, N)
-constexpr int kBinChunk = 8;                              // bins a thread sums at a time (one 16-byte load per histogram row)
-constexpr int kMaxStride = (kMaxBins + kBinChunk - 1) / kBinChunk * kBinChunk;
-constexpr int kMaxSortBlocks = 1024;
+constexpr int kBinChunk = 8;                              // bins per 16-byte load of a histogram row
+constexpr int kMaxWidth = ((kMaxBins + kSlices - 1) / kSlices + kBinChunk - 1) / kBinChunk * kBinChunk;   // bins per slice: 520
+constexpr int kMaxSortTiles = 1024;
 constexpr int kMaxTile = 63 * 1024;                       // counters are 16 bits wide
-constexpr int kRowBatch = 32;                             // histogram rows whose loads are in flight together
-static_assert(kMaxBins <= kSortThreads * kBinChunk + 1, "the scan covers 8 bins per thread plus one");
+constexpr int kRowBatch = 8;                              // histogram rows a thread has in flight
+constexpr int kGroup = 8;                                 // steps of 64 items whose loads are issued together
+static_assert(kSlices == kSortWaves, "the count kernel sums slice w in wave w");
 
 struct SortPass {
   const int32_t* keys_in;   // expert ids, in the order left by the previous pass
@@ -42,11 +48,12 @@ struct SortPass {
   int32_t* vals_out;
   int32_t* tok_out;         // NULL, or pair id / top_k (last pass)
   int32_t* offsets_out;     // NULL, or [bins]: first output position of every bin (single pass: the segment offsets)
-  uint16_t* hist;           // [blocks][stride] bin counts of every tile
+  uint16_t* hist;           // [tiles][stride] bin counts of every tile
+  uint32_t* slice_tot;      // [tiles][8] the same counts summed over each slice
   int64_t num_pairs;
-  int tile;                 // pairs per block, a multiple of 1024
-  int blocks, bins, stride, bits;   // stride = bins rounded up to 8; bits = ceil(log2(bins))
-  int sub;                  // scatter blocks per tile (a power of two that divides tile / 8)
+  int tile;                 // pairs per tile, a multiple of 1024
+  int tiles, bins;
+  int width, stride;        // bins per slice (a multiple of 8); stride = 8 * width >= bins
   int shift;                // digit = id >> shift ...
   uint32_t mask;            //   ... & mask (0xFFFFFFFF on the last pass)
   int last;                 // last pass: ids outside [0, N) go to bin bins-1; earlier passes: to bin 0
@@ -60,68 +67,75 @@ __device__ __forceinline__ int sort_digit(const SortPass& a, int32_t key) {
   return valid ? d : (a.last ? a.bins - 1 : 0);
 }
 
+__device__ __forceinline__ int32_t wave_sum_i32(int32_t v) {
+#pragma unroll
+  for (int m = kWave / 2; m >= 1; m >>= 1) v += __shfl_xor(v, m, kWave);
+  return v;
+}
+
 __global__ __launch_bounds__(kSortThreads) void sort_count_kernel(const SortPass a) {
-  extern __shared__ int32_t cnt[];
+  extern __shared__ int32_t cnt[];                       // [stride]
   for (int d = threadIdx.x; d < a.stride; d += kSortThreads) cnt[d] = 0;
   __syncthreads();
   const int64_t t0 = (int64_t)blockIdx.x * a.tile;
   const int64_t t1 = t0 + a.tile < a.num_pairs ? t0 + a.tile : a.num_pairs;
-  constexpr int kBatch = 8;                              // loads in flight per thread
-  for (int64_t i0 = t0 + threadIdx.x; i0 < t1; i0 += kBatch * kSortThreads) {
-    int32_t key[kBatch];
-#pragma unroll
-    for (int u = 0; u < kBatch; ++u) {
-      const int64_t i = i0 + u * kSortThreads;
-      key[u] = i < t1 ? a.keys_in[i] : 0;
-    }
-#pragma unroll
-    for (int u = 0; u < kBatch; ++u)
-      if (i0 + u * kSortThreads < t1) atomicAdd(&cnt[sort_digit(a, key[u])], 1);
-  }
-  __syncthreads();
-  for (int d = threadIdx.x; d < a.stride; d += kSortThreads) a.hist[(int64_t)blockIdx.x * a.stride + d] = (uint16_t)cnt[d];
-}
-
-__global__ __launch_bounds__(kSortThreads) void sort_scatter_kernel(const SortPass a) {
-  extern __shared__ int32_t tbl[];                       // [waves][stride]: counts, then running output positions; then [stride] bin bases
-  __shared__ int32_t wave_tot[kSortWaves];
-  int32_t* bin_base = tbl + kSortWaves * a.stride;
-  const int lane = lane_id(), wave = threadIdx.x >> 6;
-  // The histogram rows come from other blocks' writes, i.e. from memory: thread t takes bins 8t .. 8t+7 of every row
-  // (one 16-byte load per row), kRowBatch rows in flight together, the first batch while the tile is being counted.
-  const int d0 = threadIdx.x * kBinChunk;
-  const bool active = d0 < a.stride && d0 < kSortThreads * kBinChunk;
-  auto load_rows = [&](u32x4_t (&row)[kRowBatch], int first) {
-#pragma unroll
-    for (int j = 0; j < kRowBatch; ++j)
-      row[j] = (active && first + j < a.blocks) ? *(const u32x4_t*)(a.hist + (int64_t)(first + j) * a.stride + d0) : u32x4_t{0, 0, 0, 0};
-  };
-  u32x4_t early[kRowBatch];
-  load_rows(early, 0);
-  for (int d = threadIdx.x * 4; d < a.stride * (kSortWaves + 1); d += kSortThreads * 4) *(u32x4_t*)(tbl + d) = u32x4_t{0, 0, 0, 0};   // stride % 8 == 0
-  __syncthreads();
-  // a.sub blocks share a tile (the scattered stores are bound by the requests one CU can issue, so they are spread
-  // over many CUs); block sb of a tile places the sb-th part of it, after the parts before it
-  const int tile_idx = (int)blockIdx.x / a.sub, sb = (int)blockIdx.x % a.sub;
-  const int64_t t0 = (int64_t)tile_idx * a.tile;
-  const int64_t t1 = t0 + a.tile < a.num_pairs ? t0 + a.tile : a.num_pairs;
-  const int share = a.tile / a.sub, per_wave = share / kSortWaves;
-  const int64_t s0 = t0 + (int64_t)sb * share < t1 ? t0 + (int64_t)sb * share : t1;             // earlier parts of the tile: [t0, s0)
-  const int64_t w0 = s0 + (int64_t)wave * per_wave < t1 ? s0 + (int64_t)wave * per_wave : t1;   // this wave's eighth of the part, in order
-  const int64_t w1 = w0 + per_wave < t1 ? w0 + per_wave : t1;
-  int32_t* mine = tbl + wave * a.stride;
-  constexpr int kGroup = 8;                              // steps of 64 items whose loads are issued together
-  for (int64_t i0 = t0 + threadIdx.x; i0 < s0; i0 += kGroup * kSortThreads) {   // what the tile's earlier parts put into each bin
+  for (int64_t i0 = t0 + threadIdx.x; i0 < t1; i0 += kGroup * kSortThreads) {
     int32_t key[kGroup];
 #pragma unroll
     for (int u = 0; u < kGroup; ++u) {
       const int64_t i = i0 + u * kSortThreads;
-      key[u] = i < s0 ? a.keys_in[i] : 0;
+      key[u] = i < t1 ? a.keys_in[i] : 0;
     }
 #pragma unroll
     for (int u = 0; u < kGroup; ++u)
-      if (i0 + u * kSortThreads < s0) atomicAdd(&bin_base[sort_digit(a, key[u])], 1);
+      if (i0 + u * kSortThreads < t1) atomicAdd(&cnt[sort_digit(a, key[u])], 1);
   }
+  __syncthreads();
+  for (int c = threadIdx.x; c < a.stride / kBinChunk; c += kSortThreads) {    // 8 counters per 16-byte store
+    const int32_t* v = cnt + c * kBinChunk;
+    *(u32x4_t*)(a.hist + (int64_t)blockIdx.x * a.stride + c * kBinChunk) =
+        u32x4_t{(uint32_t)v[0] | ((uint32_t)v[1] << 16), (uint32_t)v[2] | ((uint32_t)v[3] << 16),
+                (uint32_t)v[4] | ((uint32_t)v[5] << 16), (uint32_t)v[6] | ((uint32_t)v[7] << 16)};
+  }
+  const int lane = lane_id(), wave = threadIdx.x >> 6;   // wave w sums slice w
+  int32_t sum = 0;
+  for (int d = lane; d < a.width; d += kWave) sum += cnt[wave * a.width + d];
+  sum = wave_sum_i32(sum);
+  if (lane == 0) a.slice_tot[(int64_t)blockIdx.x * kSlices + wave] = (uint32_t)sum;
+}
+
+__global__ __launch_bounds__(kSortThreads) void sort_scatter_kernel(const SortPass a) {
+  __shared__ int32_t tbl[kSortWaves][kMaxWidth];         // per wave and bin: count, then running output position
+  __shared__ int32_t bin_base[kMaxWidth], before_s[kMaxWidth], total_s[kMaxWidth];
+  __shared__ int32_t below_s;                            // pairs in the slices below this one, all tiles
+  const int lane = lane_id(), wave = threadIdx.x >> 6;
+  const int tile_idx = (int)blockIdx.x / kSlices, slice = (int)blockIdx.x % kSlices;
+  const int lo = slice * a.width;                        // this block's bins: lo .. lo + width - 1
+  // The histogram rows come from other blocks' writes, i.e. from memory.  Thread t sums chunk t % C (8 bins, one
+  // 16-byte load per row) of the rows t / C, t / C + G, ..; the first batch of loads flies while the tile is counted.
+  const int C = a.width / kBinChunk, G = kSortThreads / C;
+  const int chunk = threadIdx.x % C, group = threadIdx.x / C;
+  const bool summing = group < G;
+  auto load_rows = [&](u32x4_t (&row)[kRowBatch], int first) {
+#pragma unroll
+    for (int j = 0; j < kRowBatch; ++j) {
+      const int r = first + j * G;
+      row[j] = (summing && r < a.tiles) ? *(const u32x4_t*)(a.hist + (int64_t)r * a.stride + lo + chunk * kBinChunk) : u32x4_t{0, 0, 0, 0};
+    }
+  };
+  u32x4_t early[kRowBatch];
+  load_rows(early, group);
+  for (int d = threadIdx.x; d < kSortWaves * kMaxWidth; d += kSortThreads) (&tbl[0][0])[d] = 0;
+  for (int d = threadIdx.x; d < a.width; d += kSortThreads) bin_base[d] = before_s[d] = total_s[d] = 0;
+  if (threadIdx.x == 0) below_s = 0;
+  __syncthreads();
+
+  const int64_t t0 = (int64_t)tile_idx * a.tile;
+  const int64_t t1 = t0 + a.tile < a.num_pairs ? t0 + a.tile : a.num_pairs;
+  const int per_wave = a.tile / kSortWaves;
+  const int64_t w0 = t0 + (int64_t)wave * per_wave < t1 ? t0 + (int64_t)wave * per_wave : t1;   // this wave's eighth, in order
+  const int64_t w1 = w0 + per_wave < t1 ? w0 + per_wave : t1;
+  int32_t* mine = tbl[wave];
   for (int64_t g0 = w0; g0 < w1; g0 += kGroup * kWave) {
     int32_t key[kGroup];
 #pragma unroll
@@ -130,102 +144,95 @@ __global__ __launch_bounds__(kSortThreads) void sort_scatter_kernel(const SortPa
       key[u] = i < w1 ? a.keys_in[i] : 0;
     }
 #pragma unroll
-    for (int u = 0; u < kGroup; ++u)
-      if (g0 + u * kWave + lane < w1) atomicAdd(&mine[sort_digit(a, key[u])], 1);
+    for (int u = 0; u < kGroup; ++u) {
+      const int d = sort_digit(a, key[u]) - lo;
+      if (g0 + u * kWave + lane < w1 && (uint32_t)d < (uint32_t)a.width) atomicAdd(&mine[d], 1);
+    }
+  }
+
+  // what the slices below this one hold, over all tiles
+  {
+    int32_t part = 0;
+    for (int e = threadIdx.x; e < a.tiles * kSlices; e += kSortThreads)
+      part += (e % kSlices) < slice ? (int32_t)a.slice_tot[e] : 0;
+    part = wave_sum_i32(part);
+    if (lane == 0 && part) atomicAdd(&below_s, part);
+  }
+  // this slice of the histogram rows: what earlier tiles put into each bin, and each bin's total
+  {
+    int32_t before[kBinChunk], rest[kBinChunk];
+#pragma unroll
+    for (int i = 0; i < kBinChunk; ++i) before[i] = rest[i] = 0;
+    auto add_rows = [&](const u32x4_t (&row)[kRowBatch], int first) {
+      auto add = [&](int32_t (&acc)[kBinChunk], const u32x4_t& r) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          acc[2 * i] += (int32_t)(r[i] & 0xffffu);
+          acc[2 * i + 1] += (int32_t)(r[i] >> 16);
+        }
+      };
+#pragma unroll
+      for (int j = 0; j < kRowBatch; ++j) {
+        if (first + j * G < tile_idx) add(before, row[j]);
+        else add(rest, row[j]);                            // rows past the last tile were loaded as zeros
+      }
+    };
+    add_rows(early, group);
+    for (int r0 = group + kRowBatch * G; r0 < a.tiles; r0 += kRowBatch * G) {
+      u32x4_t row[kRowBatch];
+      load_rows(row, r0);
+      add_rows(row, r0);
+    }
+    if (summing) {
+#pragma unroll
+      for (int i = 0; i < kBinChunk; ++i) {
+        if (before[i]) atomicAdd(&before_s[chunk * kBinChunk + i], before[i]);
+        if (before[i] + rest[i]) atomicAdd(&total_s[chunk * kBinChunk + i], before[i] + rest[i]);
+      }
+    }
   }
   __syncthreads();
 
-  // Output bases.  The rows above this block's give what earlier tiles put into each bin, all rows the bin's total.
-  // An exclusive scan of the totals over the bins (thread order = bin order) gives each bin's first position.
-  // 512 threads cover 4096 bins; the one bin beyond them (ids outside the table, when there are 4096 experts) is
-  // summed by wave 0, a row per lane.
-  int32_t before[kBinChunk], rest[kBinChunk];
-#pragma unroll
-  for (int i = 0; i < kBinChunk; ++i) before[i] = rest[i] = 0;
-  auto add_rows = [&](const u32x4_t (&row)[kRowBatch], int first) {
-    auto add = [&](int32_t (&acc)[kBinChunk], const u32x4_t& r) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        acc[2 * i] += (int32_t)(r[i] & 0xffffu);
-        acc[2 * i + 1] += (int32_t)(r[i] >> 16);
-      }
-    };
-#pragma unroll
-    for (int j = 0; j < kRowBatch; ++j) {
-      if (first + j < tile_idx) add(before, row[j]);      // a scalar branch: the row index is uniform
-      else add(rest, row[j]);
-    }
-  };
-  add_rows(early, 0);
-  for (int b0 = kRowBatch; b0 < a.blocks; b0 += kRowBatch) {
-    u32x4_t row[kRowBatch];
-    load_rows(row, b0);
-    add_rows(row, b0);
-  }
-  const int tail_bin = kSortThreads * kBinChunk;         // 4096
-  int32_t tail_before = 0, tail_total = 0;
-  if (a.bins > tail_bin && wave == 0) {
-    for (int b = lane; b < a.blocks; b += kWave) {
-      const int32_t c = a.hist[(int64_t)b * a.stride + tail_bin];
-      tail_total += c;
-      tail_before += b < tile_idx ? c : 0;
-    }
-#pragma unroll
-    for (int m = kWave / 2; m >= 1; m >>= 1) {
-      tail_total += __shfl_xor(tail_total, m, kWave);
-      tail_before += __shfl_xor(tail_before, m, kWave);
-    }
-  }
-  {
-    int32_t tsum = 0;
-#pragma unroll
-    for (int i = 0; i < kBinChunk; ++i) tsum += before[i] + rest[i];
-    int32_t inc = tsum;                                  // inclusive scan across the wave
+  // exclusive scan of the slice's totals (wave 0, a run of consecutive bins per lane): every bin's first position
+  if (wave == 0) {
+    const int per = (a.width + kWave - 1) / kWave, b0 = lane * per;
+    int32_t sum = 0;
+    for (int i = 0; i < per; ++i) sum += b0 + i < a.width ? total_s[b0 + i] : 0;
+    int32_t inc = sum;
 #pragma unroll
     for (int d = 1; d < kWave; d <<= 1) {
       const int32_t o = __shfl_up(inc, d, kWave);
       if (lane >= d) inc += o;
     }
-    if (lane == kWave - 1) wave_tot[wave] = inc;
-    __syncthreads();
-    int32_t excl = inc - tsum, all = 0;
-#pragma unroll
-    for (int w = 0; w < kSortWaves; ++w) {
-      excl += w < wave ? wave_tot[w] : 0;
-      all += wave_tot[w];
-    }
-#pragma unroll
-    for (int i = 0; i < kBinChunk; ++i) {
-      const int d = d0 + i;
-      if (active && d < a.bins) {
-        if (a.offsets_out && blockIdx.x == 0) a.offsets_out[d] = excl;
-        bin_base[d] += excl + before[i];                   // on top of the earlier parts' count
+    int32_t excl = below_s + inc - sum;
+    for (int i = 0; i < per; ++i) {
+      const int b = b0 + i;
+      if (b < a.width) {
+        if (a.offsets_out && tile_idx == 0 && lo + b < a.bins) a.offsets_out[lo + b] = excl;
+        bin_base[b] = excl + before_s[b];
+        excl += total_s[b];
       }
-      excl += before[i] + rest[i];
     }
-    if (a.bins > tail_bin && threadIdx.x == 0) {         // the bin behind all others starts where they end
-      if (a.offsets_out && blockIdx.x == 0) a.offsets_out[tail_bin] = all;
-      bin_base[tail_bin] += all + tail_before;
-    }
-    __syncthreads();
   }
+  __syncthreads();
   // per-wave bases: consecutive threads take consecutive bins (no bank conflicts), wave by wave down the table
-  for (int d = threadIdx.x; d < a.bins; d += kSortThreads) {
+  for (int d = threadIdx.x; d < a.width; d += kSortThreads) {
     int32_t base = bin_base[d];
 #pragma unroll
     for (int w = 0; w < kSortWaves; ++w) {
-      const int32_t c = tbl[w * a.stride + d];
-      tbl[w * a.stride + d] = base;
+      const int32_t c = tbl[w][d];
+      tbl[w][d] = base;
       base += c;
     }
   }
   __syncthreads();
 
-  // Placement, 64 consecutive items at a time and in order.  Position = the bin's running base + the number of earlier
-  // lanes of the step with the same bin.  Every lane reads the base, then bumps it; a lane that finds the base already
-  // bumped shares its bin with another lane of its step, and only then are the lanes of that bin ranked by lane number
-  // (whatever order the adds took effect in).  LDS executes a wave's instructions in order, so the reads and adds of all
-  // steps of a group are issued back to back (a later step sees the earlier steps' adds) and waited for once.
+  // Placement, 64 consecutive items at a time and in order; only the items of this block's slice take part.
+  // Position = the bin's running base + the number of earlier lanes of the step with the same bin.  Every lane
+  // reads the base, then bumps it; a lane that finds the base already bumped shares its bin with another lane of
+  // its step, and only then are the lanes of that bin ranked by lane number (whatever order the adds took effect
+  // in).  LDS executes a wave's instructions in order, so the reads and adds of all steps of a group are issued
+  // back to back (a later step sees the earlier steps' adds) and waited for once.
   const uint64_t below = (1ull << lane) - 1ull;
   for (int64_t g0 = w0; g0 < w1; g0 += kGroup * kWave) {
     int32_t keys[kGroup], vals[kGroup], dig[kGroup], pos[kGroup], bumped[kGroup];
@@ -237,24 +244,26 @@ __global__ __launch_bounds__(kSortThreads) void sort_scatter_kernel(const SortPa
     }
 #pragma unroll
     for (int u = 0; u < kGroup; ++u) {
-      const bool active = g0 + u * kWave + lane < w1;
-      dig[u] = active ? sort_digit(a, keys[u]) : 0;
+      dig[u] = sort_digit(a, keys[u]) - lo;
+      const bool active = g0 + u * kWave + lane < w1 && (uint32_t)dig[u] < (uint32_t)a.width;
       pos[u] = bumped[u] = 0;
       if (active) {
         pos[u] = mine[dig[u]];
         bumped[u] = atomicAdd(&mine[dig[u]], 1);
+      } else {
+        dig[u] = -1;
       }
     }
 #pragma unroll
     for (int u = 0; u < kGroup; ++u) {
-      const bool active = g0 + u * kWave + lane < w1;
       const int d = dig[u];
+      const bool active = d >= 0;
       uint64_t shared = __ballot(active && bumped[u] != pos[u]);   // the non-first lanes of shared bins
       while (shared) {
         const int l = __builtin_ctzll(shared);
         const int v = __shfl(d, l, kWave);
-        const uint64_t grp = __ballot(active && d == v);           // all lanes of that bin; they read the same base
-        if (active && d == v) pos[u] += __popcll(grp & below);
+        const uint64_t grp = __ballot(d == v);                     // all lanes of that bin; they read the same base
+        if (d == v) pos[u] += __popcll(grp & below);
         shared &= ~grp;
       }
       if (active) {
@@ -285,7 +294,7 @@ static inline int ceil_log2(uint64_t v) { int b = 0; while ((1ull << b) < v) ++b
 
 // How the sort of P pairs with ids below N is split into passes and tiles.
 struct SortPlan {
-  int passes, lo_bits, bins[2], stride, tile, blocks, sub;
+  int passes, lo_bits, bins[2], width, stride, tile, tiles;
   size_t hist_entries;
 };
 static bool make_plan(int64_t P, int64_t N, SortPlan* pl) {
@@ -298,37 +307,31 @@ static bool make_plan(int64_t P, int64_t N, SortPlan* pl) {
   }
   const int maxb = pl->bins[0] > pl->bins[1] ? pl->bins[0] : pl->bins[1];
   if (maxb > kMaxBins) return false;                       // N > 16 Mi experts
-  pl->stride = (maxb + kBinChunk - 1) / kBinChunk * kBinChunk;
-  // every scatter block sums the whole histogram, one 16-byte load per row and thread: 32 rows (tiles) are one batch of
-  // loads; more only where a tile would outgrow its 16-bit counters
-  constexpr int want = 32;
-  int64_t tile = (P + want - 1) / want;
-  tile = (tile + 1023) / 1024 * 1024;
-  if (tile < 1024) tile = 1024;
+  pl->width = ((maxb + kSlices - 1) / kSlices + kBinChunk - 1) / kBinChunk * kBinChunk;
+  pl->stride = pl->width * kSlices;
+  // a wave places an eighth of a tile, 64 items a step: tiles of 8192 pairs are 16 steps; at most 256 tiles (a scatter
+  // block sums its slice of every tile's row), more only where a tile would outgrow its 16-bit counters
+  int64_t tile = 8192;
+  if ((P + tile - 1) / tile > 256) tile = ((P + 255) / 256 + 1023) / 1024 * 1024;
   if (tile > kMaxTile) tile = kMaxTile;
-  if ((P + tile - 1) / tile > kMaxSortBlocks) return false;   // more than 64 Mi pairs
+  if ((P + tile - 1) / tile > kMaxSortTiles) return false;   // more than 64 Mi pairs
   pl->tile = (int)tile;
-  pl->blocks = (int)((P + tile - 1) / tile);
-  if (pl->blocks < 1) pl->blocks = 1;
-  pl->hist_entries = (size_t)pl->stride * pl->blocks;
-  // scatter blocks per tile: towards one block per CU, each part at least 8 waves x 64 items (tile is a multiple of 1024)
-  pl->sub = 1;
-  while (pl->sub < 8 && pl->blocks * pl->sub * 2 <= 256 && pl->tile / (pl->sub * 2) >= 512) pl->sub *= 2;
+  pl->tiles = (int)((P + tile - 1) / tile);
+  if (pl->tiles < 1) pl->tiles = 1;
+  pl->hist_entries = (size_t)pl->stride * pl->tiles;
   return true;
 }
 
-// up to 9 x 4104 counters exceed the 64 KiB default
-static LdsKernel g_scatter_lds{(const void*)sort_scatter_kernel, kMaxStride * (kSortWaves + 1) * 4};
-
 }  // namespace omni
 
-// workspace: hist [blocks][stride] | two-pass sorts only: keys A [P] | keys B [P] | pair ids [P]
+// workspace: hist [tiles][stride] u16 | slice sums [tiles][8] u32 | two-pass sorts only: keys A [P] | keys B [P] | pair ids [P]
 extern "C" OMNI_API size_t omni_schedule_workspace_bytes(int64_t num_tokens, int32_t num_experts_per_token, int64_t num_experts) {
   using namespace omni;
   const int64_t P = num_tokens * (int64_t)num_experts_per_token;
   SortPlan pl;
   if (num_tokens < 0 || num_experts_per_token < 0 || num_experts <= 0 || !make_plan(P, num_experts, &pl)) return 0;
-  return align_up(pl.hist_entries * 2, 256) + (pl.passes == 2 ? 3 * align_up((size_t)P * 4 + 4, 256) : 0);
+  return align_up(pl.hist_entries * 2, 256) + align_up((size_t)pl.tiles * kSlices * 4, 256) +
+         (pl.passes == 2 ? 3 * align_up((size_t)P * 4 + 4, 256) : 0);
 }
 
 extern "C" OMNI_API int32_t omni_schedule(const int32_t* indices, int32_t* offsets, int32_t* sorted_pair_ids,
@@ -344,11 +347,11 @@ extern "C" OMNI_API int32_t omni_schedule(const int32_t* indices, int32_t* offse
   hipStream_t s = (hipStream_t)stream;
   char* w = (char*)workspace;
   uint16_t* hist = (uint16_t*)w;     w += align_up(pl.hist_entries * 2, 256);
+  uint32_t* slice_tot = (uint32_t*)w; w += align_up((size_t)pl.tiles * kSlices * 4, 256);
   int32_t* keys_a = (int32_t*)w;     w += align_up((size_t)P * 4 + 4, 256);      // the three arrays exist for two-pass sorts only
   int32_t* keys_b = (int32_t*)w;     w += align_up((size_t)P * 4 + 4, 256);
   int32_t* vals_a = (int32_t*)w;
 
-  if (hipError_t e = g_scatter_lds.ensure(); e != hipSuccess) return OMNI_ERR_HIP_BASE + (int)e;
   const bool single = pl.passes == 1;
   if (single || P > 0) {
     for (int pass = 0; pass < pl.passes; ++pass) {
@@ -361,20 +364,20 @@ extern "C" OMNI_API int32_t omni_schedule(const int32_t* indices, int32_t* offse
       a.tok_out = last ? sorted_token_ids : nullptr;
       a.offsets_out = single ? offsets : nullptr;          // one bin per expert: the bins' first positions ARE the offsets
       a.hist = hist;
+      a.slice_tot = slice_tot;
       a.num_pairs = P;
       a.tile = pl.tile;
-      a.blocks = pl.blocks;
-      a.sub = pl.sub;
+      a.tiles = pl.tiles;
       a.bins = pl.bins[pass];
+      a.width = pl.width;
       a.stride = pl.stride;
-      a.bits = ceil_log2((uint64_t)a.bins);
       a.shift = pass == 0 ? 0 : pl.lo_bits;
       a.mask = (pl.passes == 2 && pass == 0) ? (uint32_t)((1 << pl.lo_bits) - 1) : 0xFFFFFFFFu;
       a.last = last ? 1 : 0;
       a.num_experts = (uint32_t)N;
       a.inv_top_k = num_experts_per_token > 0 ? ((1ull << 40) + num_experts_per_token - 1) / (uint64_t)num_experts_per_token : 0;
-      hipLaunchKernelGGL(sort_count_kernel, dim3(a.blocks), dim3(kSortThreads), (size_t)a.stride * 4, s, a);
-      hipLaunchKernelGGL(sort_scatter_kernel, dim3(a.blocks * a.sub), dim3(kSortThreads), (size_t)a.stride * (kSortWaves + 1) * 4, s, a);
+      hipLaunchKernelGGL(sort_count_kernel, dim3(a.tiles), dim3(kSortThreads), (size_t)a.stride * 4, s, a);
+      hipLaunchKernelGGL(sort_scatter_kernel, dim3(a.tiles * kSlices), dim3(kSortThreads), 0, s, a);
     }
   }
   if (!single) {
