@@ -41,8 +41,8 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 # Bytes that cross the fabric per launch (FETCH_SIZE + WRITE_SIZE of rocprofv3 --pmc, each scaled by a plain copy of
 # known size); counters cannot be read in-process, so these are the figures of the committed summaries named here.
 TRAFFIC_SOURCE = "profiles/bench_layer_c4_hbm_counters.txt, profiles/expert_c5_hbm_counters.txt"
-TRAFFIC_BYTES = {"expert_c3": 182.8e6, "expert_c4": 57.8e6, "expert_gather_c3": 898.5e6, "gateup_c4": 134.7e6, "down_c4": 117.6e6,
-                 "down_plain_c4": 109.2e6, "schedule_c3": 13.34e6,
+TRAFFIC_BYTES = {"expert_c3": 182.4e6, "expert_c4": 57.8e6, "expert_gather_c3": 897.7e6, "gateup_c4": 134.7e6, "down_c4": 117.6e6,
+                 "down_plain_c4": 109.2e6, "schedule_c3": 12.36e6,
                  "expert_c5_routed": 1029.2e6, "expert_c5_uniform": 8846.8e6}
 SECTIONS = ("layer", "kernels", "expert_c3", "expert_c5", "probe", "train", "cpu")
 
@@ -305,7 +305,7 @@ def main():
         m, b = time_launches(torch, lambda: hip.hip_omni_schedule_func(i3, N))
         kernels.append(hbm_entry("schedule (stable counting sort of the pairs by expert: sort_count_kernel + sort_scatter_kernel), c3", m, b,
                                  T3 * k * 12 + 4 * (N + 1), TRAFFIC_BYTES["schedule_c3"],
-                                 note="ids in, pair ids + token ids + offsets out; bounded by per-block work on the 4097-bin tables, not by bytes"))
+                                 note="ids in, pair ids + token ids + offsets out; writes equal the algorithmic 2.1 MB (every output line goes through one L2), the ids are fetched by all 8 XCDs"))
         m, b = time_launches(torch, lambda: hip.hip_omni_expert_func(x3, up3, down3, g3, i3, algo="segment"))
         kernels.append(hbm_entry("expert op, expert-centric 'segment' algorithm (schedule + scores pass + token pass), c3", m, b,
                                  expert_alg_bytes(T3, H, k), note="for comparison; same results as the gather algorithm"))

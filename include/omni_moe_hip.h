@@ -100,7 +100,7 @@ OMNI_API int32_t omni_schedule(const int32_t* indices, int32_t* offsets, int32_t
  * omni_schedule, without the workspace: the sort's scratch is a fixed array of
  * OMNI_SCHEDULE_NOALLOC_SCRATCH_BYTES that every GPU the library runs on holds until the process ends.
  * The call allocates and frees nothing.  Requests whose omni_schedule_workspace_bytes() exceeds the
- * array return OMNI_ERR_SCRATCH (nothing enqueued); up to 65 million pairs fit when num_experts <= 4096 (one counting pass: only the histogram lives there), about 680 000 pairs above that (two passes keep three arrays of pairs).
+ * array return OMNI_ERR_SCRATCH (nothing enqueued); about 64 million pairs fit when num_experts <= 4096 (one counting pass: only the histograms live there), about 690 000 pairs above that (two passes keep three arrays of pairs).
  * All calls on one GPU share that GPU's array: calls that may overlap on the device (different
  * streams without an ordering between them) race; calls on one stream are safe. */
 #define OMNI_SCHEDULE_NOALLOC_SCRATCH_BYTES (8u << 20)
