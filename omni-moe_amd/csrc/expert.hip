@@ -369,34 +369,42 @@ __global__ __launch_bounds__(kTokensPerBlock* kWave) void expert_split_accumulat
   for (int i = 0; i < E; ++i) acc[i] = 0.f;
   for (int jb = 0; jb < top_k; jb += LPR) {
     const int j = jb + sub;
-    float coef = 0.f;
     int my_id = -1;                                               // -1: a padded slot or an id outside the table
     if (j < top_k) {
+      const int id = ids[base + j];
+      if ((uint32_t)id < num_experts) my_id = id;
+    }
+    // the down rows only need the ids: their loads are issued ahead of the partial sums the coefficients wait for
+    u32x4_t vr[LPR];
+    bool used[LPR];
+#pragma unroll
+    for (int e = 0; e < LD; ++e) {
+      const int id = __shfl(my_id, grp * LPR + e, kWave);         // from the lane of this group that holds pair e
+      used[e] = id >= 0;
+      vr[e] = *(const u32x4_t*)(down + int64_t(used[e] ? id : 0) * row_bytes + col);
+    }
+    float coef = 0.f;
+    if (my_id >= 0) {
       float sdot = 0.f;
 #pragma unroll
       for (int sl = 0; sl < kSlices; ++sl) sdot += partial[(int64_t(sl) * num_tokens + tt) * top_k + j];
-      const int id = ids[base + j];
-      if ((uint32_t)id < num_experts) {
-        my_id = id;
-        coef = silu_f32(sdot) * Elem<DT>::load(gates, base + j);
-      }
+      coef = silu_f32(sdot) * Elem<DT>::load(gates, base + j);
     }
 #pragma unroll
     for (int e0 = 0; e0 < LPR; e0 += LD) {
-      u32x4_t vr[LD];
-      float cf[LD];
-      bool used[LD];
+      if (e0 + LD < LPR) {
 #pragma unroll
-      for (int e = 0; e < LD; ++e) {
-        const int src = grp * LPR + e0 + e;                       // the lane of this group that holds pair e0+e
-        const int id = __shfl(my_id, src, kWave);
-        cf[e] = __shfl(coef, src, kWave);
-        used[e] = id >= 0;
-        vr[e] = *(const u32x4_t*)(down + int64_t(used[e] ? id : 0) * row_bytes + col);
+        for (int e = 0; e < LD; ++e) {
+          const int id = __shfl(my_id, grp * LPR + e0 + LD + e, kWave);
+          used[e0 + LD + e] = id >= 0;
+          vr[e0 + LD + e] = *(const u32x4_t*)(down + int64_t(used[e0 + LD + e] ? id : 0) * row_bytes + col);
+        }
       }
 #pragma unroll
-      for (int e = 0; e < LD; ++e)
-        if (used[e]) axpy16<DT>(cf[e], vr[e], acc);             // not even 0 * row: the stand-in row may hold Inf or NaN
+      for (int e = 0; e < LD; ++e) {
+        const float cf = __shfl(coef, grp * LPR + e0 + e, kWave);
+        if (used[e0 + e]) axpy16<DT>(cf, vr[e0 + e], acc);        // not even 0 * row: the stand-in row may hold Inf or NaN
+      }
     }
   }
   if (live) *(u32x4_t*)(y + t * row_bytes + col) = pack16<DT>(acc);
