@@ -90,7 +90,9 @@ def test_router_select_contract(device):
 # ---------------------------------------------------------------- schedule
 SCHED_CASES = [(512, 8, 1024, "uniform"), (4096, 16, 4096, "uniform"), (16384, 16, 4096, "uniform"),
                (4096, 32, 262144, "zipf"), (1000, 6, 5000, "zipf"), (3, 2, 7, "uniform"), (2048, 16, 64, "hot"),
-               (32768, 32, 262144, "zipf"), (777, 10, 1048576, "uniform"), (100, 4, 1, "hot"), (5000, 8, 4097, "uniform")]
+               (32768, 32, 262144, "zipf"), (777, 10, 1048576, "uniform"), (100, 4, 1, "hot"), (5000, 8, 4097, "uniform"),
+               # more than 256 tiles of 8192 pairs (tiles grow), and tiles at their 16-bit limit with every pair in one bin
+               (150000, 16, 4096, "uniform"), (1100000, 16, 4096, "hot")]
 
 
 def _sched_ids(T, k, N, kind, seed):
