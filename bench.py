@@ -266,10 +266,17 @@ def main():
         r = layer.num_expert_sqrt
         m, b = time_launches(torch, lambda: hip.hip_swiglu_linear_func(xf, layer.gate_proj.weight, layer.up_proj.weight))
         kernels.append(mfma_entry("gemm_nt_dma_kernel<swiglu> (gate/up projection + SwiGLU), c4", 4 * T * H * I, m, b, TRAFFIC_BYTES["gateup_c4"], sustained))
+        # for orientation: the vendor library (torch.matmul) on the same operands, without the SwiGLU (one GEMM over [Wg; Wu])
+        wcat = torch.cat([layer.gate_proj.weight, layer.up_proj.weight], 0)
+        m_lib, b_lib = time_launches(torch, lambda: torch.matmul(xf, wcat.t()))
+        kernels[-1]["library_gemm_same_flops_ms"] = m_lib
+        m_lib, b_lib = time_launches(torch, lambda: torch.matmul(h, layer.down_proj.weight.t()))
+        del wcat
         m, b = time_launches(torch, lambda: hip.hip_linear_func(h, layer.down_proj.weight, e_out))
         kernels.append(mfma_entry("gemm_nt_dma_kernel<residual> (down projection + experts add), c4", 2 * T * H * I, m, b, TRAFFIC_BYTES["down_c4"], sustained))
         m, b = time_launches(torch, lambda: hip.hip_linear_func(h, layer.down_proj.weight))
         kernels.append(mfma_entry("gemm_nt_dma_kernel<plain> (down projection alone, as on the two-stream path), c4", 2 * T * H * I, m, b, TRAFFIC_BYTES["down_plain_c4"], sustained))
+        kernels[-1]["library_gemm_same_flops_ms"] = m_lib
         m, b = time_launches(torch, lambda: hip.hip_add_inplace_func(y0, e_out))
         kernels.append(hbm_entry("add_inplace_kernel (join of the two branches), c4", m, b, 3 * T * H * 2, resident_in_hbm=False,
                                  note="24 MiB that the caches hold between launches"))
