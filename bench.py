@@ -41,7 +41,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 # Bytes that cross the fabric per launch (FETCH_SIZE + WRITE_SIZE of rocprofv3 --pmc, each scaled by a plain copy of
 # known size); counters cannot be read in-process, so these are the figures of the committed summaries named here.
 TRAFFIC_SOURCE = "profiles/bench_layer_c4_hbm_counters.txt, profiles/expert_c5_hbm_counters.txt"
-TRAFFIC_BYTES = {"expert_c3": 180.6e6, "expert_c4": 57.8e6, "expert_gather_c3": 897.0e6, "gateup_c4": 134.7e6, "down_c4": 117.6e6,
+TRAFFIC_BYTES = {"expert_c3": 180.6e6, "expert_c4": 57.8e6, "expert_gather_c3": 897.2e6, "gateup_c4": 134.4e6, "down_c4": 117.6e6,
                  "down_plain_c4": 109.2e6, "schedule_c3": 12.36e6,
                  "expert_c5_routed": 1029.2e6, "expert_c5_uniform": 8846.8e6}
 SECTIONS = ("layer", "kernels", "expert_c3", "expert_c5", "probe", "train", "cpu")
