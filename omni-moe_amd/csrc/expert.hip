@@ -374,15 +374,17 @@ __global__ __launch_bounds__(kTokensPerBlock* kWave) void expert_split_accumulat
       const int id = ids[base + j];
       if ((uint32_t)id < num_experts) my_id = id;
     }
-    // the down rows only need the ids: their loads are issued ahead of the partial sums the coefficients wait for
-    u32x4_t vr[LPR];
-    bool used[LPR];
-#pragma unroll
-    for (int e = 0; e < LD; ++e) {
+    // the down rows only need the ids: the first LD of them are requested ahead of the partial sums the coefficients
+    // wait for; every row that has been added makes room for the request of a later one (LD row registers in all)
+    u32x4_t vr[LD];
+    bool used[LD];
+    auto request = [&](int slot, int e) {
       const int id = __shfl(my_id, grp * LPR + e, kWave);         // from the lane of this group that holds pair e
-      used[e] = id >= 0;
-      vr[e] = *(const u32x4_t*)(down + int64_t(used[e] ? id : 0) * row_bytes + col);
-    }
+      used[slot] = id >= 0;
+      vr[slot] = *(const u32x4_t*)(down + int64_t(used[slot] ? id : 0) * row_bytes + col);
+    };
+#pragma unroll
+    for (int e = 0; e < LD; ++e) request(e, e);
     float coef = 0.f;
     if (my_id >= 0) {
       float sdot = 0.f;
@@ -391,20 +393,10 @@ __global__ __launch_bounds__(kTokensPerBlock* kWave) void expert_split_accumulat
       coef = silu_f32(sdot) * Elem<DT>::load(gates, base + j);
     }
 #pragma unroll
-    for (int e0 = 0; e0 < LPR; e0 += LD) {
-      if (e0 + LD < LPR) {
-#pragma unroll
-        for (int e = 0; e < LD; ++e) {
-          const int id = __shfl(my_id, grp * LPR + e0 + LD + e, kWave);
-          used[e0 + LD + e] = id >= 0;
-          vr[e0 + LD + e] = *(const u32x4_t*)(down + int64_t(used[e0 + LD + e] ? id : 0) * row_bytes + col);
-        }
-      }
-#pragma unroll
-      for (int e = 0; e < LD; ++e) {
-        const float cf = __shfl(coef, grp * LPR + e0 + e, kWave);
-        if (used[e0 + e]) axpy16<DT>(cf, vr[e0 + e], acc);        // not even 0 * row: the stand-in row may hold Inf or NaN
-      }
+    for (int e = 0; e < LPR; ++e) {
+      const float cf = __shfl(coef, grp * LPR + e, kWave);
+      if (used[e % LD]) axpy16<DT>(cf, vr[e % LD], acc);          // not even 0 * row: the stand-in row may hold Inf or NaN
+      if (e + LD < LPR) request(e % LD, e + LD);
     }
   }
   if (live) *(u32x4_t*)(y + t * row_bytes + col) = pack16<DT>(acc);
