@@ -325,14 +325,15 @@ __global__ __launch_bounds__(kTokensPerBlock* kWave) void expert_split_dots_kern
   const u32x4_t xr = *(const u32x4_t*)(x + tt * row_bytes + col);
   const int64_t base = int64_t(tt) * top_k;
   for (int jb = 0; jb < top_k; jb += LPR) {
+    // lane `sub` of a group fetches the id of pair `sub` of the batch; the group reads the ids from its lanes
+    const int my_id = ids[base + min(jb + sub, top_k - 1)];
     float d[LPR];
 #pragma unroll
     for (int e0 = 0; e0 < LPR; e0 += LD) {
       u32x4_t ur[LD];
 #pragma unroll
       for (int e = 0; e < LD; ++e) {
-        const int j = min(jb + e0 + e, top_k - 1);
-        const int id = ids[base + j];                            // one address per group: a broadcast load
+        const int id = __shfl(my_id, grp * LPR + e0 + e, kWave);
         ur[e] = *(const u32x4_t*)(up + int64_t((uint32_t)id < num_experts ? id : 0) * row_bytes + col);
       }
 #pragma unroll
@@ -341,7 +342,7 @@ __global__ __launch_bounds__(kTokensPerBlock* kWave) void expert_split_dots_kern
     const float total = reduce_scatter_group<LPR>(d, lane);
     const int j = jb + sub;
     if (live && j < top_k) {
-      const bool ok = (uint32_t)ids[base + j] < num_experts;
+      const bool ok = (uint32_t)my_id < num_experts;
       partial[(int64_t(slice) * num_tokens + t) * top_k + j] = ok ? total : 0.f;
     }
   }
