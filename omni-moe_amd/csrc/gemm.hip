@@ -6,7 +6,8 @@
 //   * down projection     y  = h Wd^T (+ expert output)        (interface.py:23-29, omni_moe.py:102)
 //
 // Structure: a block of 4 waves (2 x 2) owns a (2*TM*32) x (2*TN*32) tile; each wave owns
-// TM x TN MFMA tiles of 32x32 and K advances 64 at a time.  16-bit operands with K % 64 == 0
+// TM x TN MFMA tiles of 32x32 and K advances 64 at a time.  The largest tile, 256 x 256, runs
+// on 8 waves (2 x 4, two per SIMD) of 128 x 64 instead.  16-bit operands with K % 64 == 0
 // take `gemm_nt_dma_kernel` (global -> LDS directly, ring of stages, swizzled rows); anything
 // else takes `gemm_nt_kernel` (global -> registers -> one of two LDS stages with padded rows).
 // The weight fragment is the MFMA's first operand, so an accumulator lane holds 4 consecutive
