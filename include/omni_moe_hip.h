@@ -165,6 +165,15 @@ OMNI_API int32_t omni_swiglu_linear_fwd(const void* x, const void* gate_weight, 
 OMNI_API int32_t omni_linear_fwd(const void* x, const void* weight, const void* residual, void* y, int64_t num_tokens,
                                  int32_t in_features, int32_t out_features, int32_t dtype, void* stream);
 
+/* omni_swiglu_linear_fwd that also keeps the two projections a backward pass needs (the reference materialises them:
+ * interface.py:23-27 calls torch.matmul twice before the SwiGLU function saves gate and up, omni_mlp.py:359-371):
+ *   gate_out, up_out [T,I]: x Wg^T and x Wu^T rounded to the storage dtype; h [T,I] their SwiGLU product.
+ * bf16 / f16 only, intermediate_size % 8 == 0, hidden_size % 64 == 0, 16-byte aligned outputs; anything else
+ * returns OMNI_ERR_UNSUPPORTED (use omni_linear_fwd twice and omni_swiglu_fwd). */
+OMNI_API int32_t omni_swiglu_linear_save_fwd(const void* x, const void* gate_weight, const void* up_weight, void* h,
+                                             void* gate_out, void* up_out, int64_t num_tokens, int32_t hidden_size,
+                                             int32_t intermediate_size, int32_t dtype, void* stream);
+
 /* Diagnostic, no counterpart in the reference: the device's matrix-core rate with nothing else going on.
  * num_blocks blocks of 4 waves each issue iters x 16 v_mfma_f32_32x32x16_bf16 (iters * 16 * 32768 flop per
  * wave) on register operands read once from `operands` (8 KiB; the bits matter: the clock the board sustains

@@ -78,6 +78,8 @@ struct GemmArgs {           // all element offsets below are scaled by the eleme
   float* part_mean;       // kEpiStats only: [ceil(M/32)][N] mean of each column over
   float* part_m2;         //   rows 32s..32s+31 of the ROUNDED result, and the sum of squared deviations
   const float* gate;      // kEpiGate only: [M, N] fp32 factors; C is then [M, 2N]: round(v) in columns 0..N-1, round(v - round(v)) in N..2N-1
+  uint8_t* save_gate;     // kEpiSwiglu only, or NULL: [M, N] the rounded gate and up projections, kept for a backward pass
+  uint8_t* save_up;       //   (16-byte stores only: N % 8 == 0)
 };
 
 // Which output tile a block owns.  Blocks go round-robin over the 8 XCDs; each XCD gets
@@ -262,6 +264,28 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, f32x16_t (&acc)
             const auto s1 = __builtin_amdgcn_permlane32_swap(w[0][1], w[1][1], false, false);
             const int n = nt + pr * 16 + (lane >> 5) * 8;
             if (n < g.N) *(u32x4_t*)(g.c + ((int64_t)m * g.N + n) * 2) = u32x4_t{s0[0], s1[0], s0[1], s1[1]};
+            if constexpr (EPI == kEpiSwiglu) {
+              if (g.save_gate) {                             // the two rounded projections leave the same way
+                uint32_t a[2][2], b[2][2];
+#pragma unroll
+                for (int e = 0; e < 2; ++e) {
+                  const int q4 = 2 * pr + e;
+#pragma unroll
+                  for (int h2 = 0; h2 < 2; ++h2) {
+                    a[e][h2] = pack2<DT>(acc[i][j][q4 * 4 + 2 * h2], acc[i][j][q4 * 4 + 2 * h2 + 1]);
+                    b[e][h2] = pack2<DT>(acc[i][j + TNO][q4 * 4 + 2 * h2], acc[i][j + TNO][q4 * 4 + 2 * h2 + 1]);
+                  }
+                }
+                const auto a0 = __builtin_amdgcn_permlane32_swap(a[0][0], a[1][0], false, false);
+                const auto a1 = __builtin_amdgcn_permlane32_swap(a[0][1], a[1][1], false, false);
+                const auto b0 = __builtin_amdgcn_permlane32_swap(b[0][0], b[1][0], false, false);
+                const auto b1 = __builtin_amdgcn_permlane32_swap(b[0][1], b[1][1], false, false);
+                if (n < g.N) {
+                  *(u32x4_t*)(g.save_gate + ((int64_t)m * g.N + n) * 2) = u32x4_t{a0[0], a1[0], a0[1], a1[1]};
+                  *(u32x4_t*)(g.save_up + ((int64_t)m * g.N + n) * 2) = u32x4_t{b0[0], b1[0], b0[1], b1[1]};
+                }
+              }
+            }
           }
           continue;
         }
@@ -636,6 +660,7 @@ static hipError_t launch_gemm(GemmArgs g, hipStream_t s) {
   g.wide = (DT != kF32) && g.N % 8 == 0 && ((uintptr_t)g.c % 16 == 0);
   g.single = g.N % 4 != 0;
   if (EPI == kEpiGate && !(g.wide && (uintptr_t)g.gate % 16 == 0)) return hipErrorInvalidValue;   // the gate epilogue has the 16-byte form only
+  if (EPI == kEpiSwiglu && g.save_gate && !g.wide) return hipErrorInvalidValue;                  // so has the saving SwiGLU epilogue
   if (blocks % 256 == 0) {
     if (g.tiles_m % 4 == 0 && g.tiles_n % 8 == 0) { g.patch_m = 4; g.patch_n = 8; }
     else if (g.tiles_m % 8 == 0 && g.tiles_n % 4 == 0) { g.patch_m = 8; g.patch_n = 4; }
@@ -704,10 +729,15 @@ static int gemm_plain(const void* a, const void* b, const void* b_hi, const void
 }
 
 template <int DT>
-static int gemm_swiglu(const void* x, const void* wg, const void* wu, void* h, int64_t M, int64_t I, int64_t K, hipStream_t s) {
+static int gemm_swiglu(const void* x, const void* wg, const void* wu, void* h, int64_t M, int64_t I, int64_t K, hipStream_t s,
+                       void* save_gate = nullptr, void* save_up = nullptr) {
   if (int e = check_gemm(M, I, K, ElemBytes<DT>::value)) return e;
   if (M == 0) return OMNI_OK;
-  GemmArgs g{(const uint8_t*)x, (const uint8_t*)wg, (const uint8_t*)wu, nullptr, (uint8_t*)h, (int)M, (int)I, (int)K, 0, 0, 0, 0, 0, 0, nullptr, nullptr, nullptr};
+  GemmArgs g{(const uint8_t*)x, (const uint8_t*)wg, (const uint8_t*)wu, nullptr, (uint8_t*)h, (int)M, (int)I, (int)K, 0, 0, 0, 0, 0, 0, nullptr, nullptr, nullptr,
+             (uint8_t*)save_gate, (uint8_t*)save_up};
+  if (save_gate) {   // the saving epilogue has the 16-byte form only, in the direct-to-LDS kernel
+    if (DT == kF32 || I % 8 != 0 || K % 64 != 0 || (uintptr_t)h % 16 || (uintptr_t)save_gate % 16 || (uintptr_t)save_up % 16) return OMNI_ERR_UNSUPPORTED;
+  }
   const int64_t big = ((M + 255) / 256) * ((I + 127) / 128);
   hipError_t err;
   if (big >= 200) err = launch_gemm<DT, 4, 4, kEpiSwiglu>(g, s);
@@ -796,6 +826,21 @@ extern "C" OMNI_API int32_t omni_swiglu_linear_fwd(const void* x, const void* ga
     case OMNI_BF16: return gemm_swiglu<kBF16>(x, gate_weight, up_weight, h, num_tokens, intermediate_size, hidden_size, s);
     case OMNI_F16: return gemm_swiglu<kF16>(x, gate_weight, up_weight, h, num_tokens, intermediate_size, hidden_size, s);
     case OMNI_F32: return gemm_swiglu<kF32>(x, gate_weight, up_weight, h, num_tokens, intermediate_size, hidden_size, s);
+    default: return OMNI_ERR_DTYPE;
+  }
+}
+
+extern "C" OMNI_API int32_t omni_swiglu_linear_save_fwd(const void* x, const void* gate_weight, const void* up_weight, void* h,
+                                                        void* gate_out, void* up_out, int64_t num_tokens, int32_t hidden_size,
+                                                        int32_t intermediate_size, int32_t dtype, void* stream) {
+  using namespace omni;
+  if (num_tokens == 0) return OMNI_OK;
+  if (!x || !gate_weight || !up_weight || !h || !gate_out || !up_out) return OMNI_ERR_NULL;
+  hipStream_t s = (hipStream_t)stream;
+  switch (dtype) {
+    case OMNI_BF16: return gemm_swiglu<kBF16>(x, gate_weight, up_weight, h, num_tokens, intermediate_size, hidden_size, s, gate_out, up_out);
+    case OMNI_F16: return gemm_swiglu<kF16>(x, gate_weight, up_weight, h, num_tokens, intermediate_size, hidden_size, s, gate_out, up_out);
+    case OMNI_F32: return OMNI_ERR_UNSUPPORTED;
     default: return OMNI_ERR_DTYPE;
   }
 }

@@ -18,7 +18,7 @@ LIB_PATH = os.path.join(_HERE, "libomni_moe_hip.so")
 
 OMNI_BF16, OMNI_F16, OMNI_F32 = 0, 1, 2
 ALGO_AUTO, ALGO_GATHER, ALGO_SEGMENT, ALGO_SPLIT, ALGO_DENSE = 0, 1, 2, 3, 4
-ERR_TOPK, ERR_SHAPE = -4, -2
+ERR_TOPK, ERR_SHAPE, ERR_UNSUPPORTED = -4, -2, -5
 
 DTYPE_CODE = {torch.bfloat16: OMNI_BF16, torch.float16: OMNI_F16, torch.float32: OMNI_F32}
 
@@ -36,6 +36,7 @@ SIGNATURES = {
     "omni_mlp_fwd": (c_int32, [c_void_p] * 6 + [c_int64, c_int32, c_int32, c_int32, c_void_p, c_void_p]),
     "omni_linear_fwd": (c_int32, [c_void_p] * 4 + [c_int64, c_int32, c_int32, c_int32, c_void_p]),
     "omni_swiglu_linear_fwd": (c_int32, [c_void_p] * 4 + [c_int64, c_int32, c_int32, c_int32, c_void_p]),
+    "omni_swiglu_linear_save_fwd": (c_int32, [c_void_p] * 6 + [c_int64, c_int32, c_int32, c_int32, c_void_p]),
     "omni_moe_workspace_bytes": (c_size_t, [c_int64, c_int32, c_int32, c_int64, c_int32, c_int32, c_int32]),
     "omni_moe_fwd": (c_int32, [c_void_p] * 15 + [c_int64, c_int32, c_int32, c_int64, c_int32, c_int32, c_int32, c_int32,
                                c_int32, c_float, c_float] + [c_void_p] * 5),

@@ -256,10 +256,15 @@ def hip_omni_mlp_func(
         tensors.append(residual)
     dev = _lib.require_gpu(*tensors)
     if _needs_grad(*tensors):
-        # the reference's composition (interface.py:23-29): three matmuls around the SwiGLU function
-        gate = OmniLinearFunc.apply(x, gate_weight)
-        up = OmniLinearFunc.apply(x, up_weight)
-        y = OmniLinearFunc.apply(OmniSwiGLUFunc.apply(gate, up), down_weight)
+        # the reference's composition (interface.py:23-29): three matmuls around the SwiGLU function.  Where the fused
+        # kernel can keep gate and up for the backward pass, the first two matmuls and the SwiGLU are one launch.
+        if _swiglu_linear_save_covers(x, gate_weight):
+            h = OmniSwiGLULinearFunc.apply(x, gate_weight, up_weight)
+        else:
+            gate = OmniLinearFunc.apply(x, gate_weight)
+            up = OmniLinearFunc.apply(x, up_weight)
+            h = OmniSwiGLUFunc.apply(gate, up)
+        y = OmniLinearFunc.apply(h, down_weight)
         return y if residual is None else y + residual
     x, gate_weight, up_weight, down_weight = (_c(t.detach()) for t in (x, gate_weight, up_weight, down_weight))
     residual = _c(residual.detach()) if residual is not None else None
@@ -352,6 +357,43 @@ def hip_swiglu_bwd_func(dout, gate, up):
                                            gate.numel(), _lib.DTYPE_CODE[gate.dtype], _lib.stream_ptr())
     _lib.check(code, "omni_swiglu_bwd")
     return dgate, dup
+
+
+def _swiglu_linear_save_covers(x, gate_weight) -> bool:
+    """Shapes the saving form of the fused gate/up GEMM takes (omni_swiglu_linear_save_fwd)."""
+    return x.dtype in (torch.bfloat16, torch.float16) and gate_weight.size(0) % 8 == 0 and x.size(1) % 64 == 0
+
+
+class OmniSwiGLULinearFunc(torch.autograd.Function):
+    """h = silu(x Wg^T) * (x Wu^T) as ONE GEMM launch that also keeps the rounded gate and up projections, which is all
+    the backward pass needs: the first three steps of ``triton_omni_mlp_func`` (reference interface.py:23-27, with
+    ``TritonSwiGLUFunc`` saving gate and up, omni_mlp.py:359-371)."""
+
+    @staticmethod
+    def forward(ctx, x, gate_weight, up_weight):
+        xd, wg, wu = _c(x.detach()), _c(gate_weight.detach()), _c(up_weight.detach())
+        T, I = xd.size(0), wg.size(0)
+        h = torch.empty(T, I, device=xd.device, dtype=xd.dtype)
+        gate, up = torch.empty_like(h), torch.empty_like(h)
+        with torch.cuda.device(xd.device):
+            code = _lib.load().omni_swiglu_linear_save_fwd(_lib.ptr(xd), _lib.ptr(wg), _lib.ptr(wu), _lib.ptr(h), _lib.ptr(gate), _lib.ptr(up),
+                                                           T, xd.size(1), I, _lib.DTYPE_CODE[xd.dtype], _lib.stream_ptr())
+        _lib.check(code, "omni_swiglu_linear_save_fwd")
+        ctx.save_for_backward(xd, wg, wu, gate, up)
+        return h
+
+    @staticmethod
+    def backward(ctx, dh):
+        x, wg, wu, gate, up = ctx.saved_tensors
+        dgate, dup = hip_swiglu_bwd_func(dh, gate, up)
+        dx = dw_g = dw_u = None
+        if ctx.needs_input_grad[0]:
+            dx = torch.addmm(dgate.matmul(wg), dup, wu)
+        if ctx.needs_input_grad[1]:
+            dw_g = dgate.t().matmul(x)
+        if ctx.needs_input_grad[2]:
+            dw_u = dup.t().matmul(x)
+        return dx, dw_g, dw_u
 
 
 class OmniSwiGLUFunc(torch.autograd.Function):

@@ -169,6 +169,36 @@ def test_swiglu_fwd_bwd(dtype, device):
         hip.hip_swiglu_func(a.to(device), b.to(device).to(torch.float16 if dtype != torch.float16 else torch.float32))
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+@pytest.mark.parametrize("shape", [(192, 128, 256), (4096, 1024, 4096), (77, 64, 136)], ids=lambda s: "T%d-H%d-I%d" % s)
+def test_swiglu_linear_save_keeps_gate_and_up(shape, dtype, device):
+    """The fused gate/up GEMM in its saving form (what the differentiable MLP op runs): gate and up are exactly the two
+    plain projections, h is exactly the non-saving fused result."""
+    from omni_moe.ops.hip import _lib
+    from omni_moe.ops.hip.interface import OmniSwiGLULinearFunc
+    T, H, I = shape
+    g = torch.Generator().manual_seed(11)
+    x = torch.randn(T, H, generator=g).to(dtype).to(device)
+    wg = (torch.randn(I, H, generator=g) * 0.05).to(dtype).to(device)
+    wu = (torch.randn(I, H, generator=g) * 0.05).to(dtype).to(device)
+    hip = _ops()
+    h = torch.empty(T, I, device=device, dtype=dtype)
+    gate, up = torch.empty_like(h), torch.empty_like(h)
+    code = _lib.load().omni_swiglu_linear_save_fwd(x.data_ptr(), wg.data_ptr(), wu.data_ptr(), h.data_ptr(), gate.data_ptr(), up.data_ptr(),
+                                                   T, H, I, _lib.DTYPE_CODE[dtype], torch.cuda.current_stream().cuda_stream)
+    assert code == 0
+    assert torch.equal(gate, hip.hip_linear_func(x, wg))
+    assert torch.equal(up, hip.hip_linear_func(x, wu))
+    assert torch.equal(h, hip.hip_swiglu_linear_func(x, wg, wu))
+    xr = x.clone().requires_grad_()
+    assert torch.equal(OmniSwiGLULinearFunc.apply(xr, wg, wu), h)
+    # fp32 storage and intermediate sizes that are not a multiple of 8 are refused (the Python op composes three launches there)
+    assert _lib.load().omni_swiglu_linear_save_fwd(x.data_ptr(), wg.data_ptr(), wu.data_ptr(), h.data_ptr(), gate.data_ptr(), up.data_ptr(),
+                                                   T, H, I, _lib.OMNI_F32, None) == _lib.ERR_UNSUPPORTED
+    assert _lib.load().omni_swiglu_linear_save_fwd(x.data_ptr(), wg.data_ptr(), wu.data_ptr(), h.data_ptr(), gate.data_ptr(), up.data_ptr(),
+                                                   T, H, I - 4, _lib.DTYPE_CODE[dtype], None) == _lib.ERR_UNSUPPORTED
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
 def test_mlp_func_autograd(dtype, device):
     """The differentiable MLP op (three GEMMs around the SwiGLU function) against fp64 autograd; its forward
