@@ -216,7 +216,7 @@ def main():
             g_med, g_best = time_launches(torch, lambda: layer(dx), n=20, reps=5, warmup=3)
         out["grad_enabled_forward"] = {"ms_per_step": g_med, "ms_per_step_best": g_best, "tokens_per_s": T / (g_med * 1e-3),
                                        "note": "moe(x) with autograd recording (README quick start): router stage, expert op and MLP op as "
-                                               "differentiable nodes, gate and up projections as separate GEMMs"}
+                                               "differentiable nodes; the gate/up GEMM also stores gate and up for the backward pass"}
 
         # correctness spot check against the oracle (outside the timed region): eval mode on both
         # sides so that the repeated train-mode steps above do not matter
