@@ -302,7 +302,7 @@ def main():
         e3 = hbm_entry("expert op (split algorithm: expert_split_dots_kernel + expert_split_accumulate_kernel), c3 (T=16384)", m, b,
                        expert_alg_bytes(T3, H, k), TRAFFIC_BYTES["expert_c3"], expert_min_bytes(T3, H, N, k),
                        note="the 16 MiB tables are cache-resident (each XCD's L2 holds the eighth of them its blocks use): the kernel is bound by "
-                            "L2 bandwidth and VALU issue, so the fraction of HBM peak counts only the bytes that cross the fabric")
+                            "the vector-memory path (L2 hits), so the fraction of HBM peak counts only the bytes that cross the fabric")
         kernels.append(e3)
         out["roofline_expert"] = e3
         m, b = time_launches(torch, lambda: hip.hip_omni_expert_func(x3, up3, down3, g3, i3, algo="gather"))
