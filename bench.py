@@ -131,7 +131,8 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=100,
+                    help="untimed steps; the first ~100 steps after the GPU has idled run about 7 %% slower (clocks ramp up)")
     ap.add_argument("--sections", default=",".join(SECTIONS), help="comma-separated subset of: " + ", ".join(SECTIONS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernels", action="store_true", help="only the layer steps (profiling runs)")
