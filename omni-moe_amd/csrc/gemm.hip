@@ -672,19 +672,20 @@ static hipError_t launch_gemm(GemmArgs g, hipStream_t s) {
   if constexpr (DT != kF32) if (g.K % kDmaBK == 0) {
     constexpr int kDmaLds = kDmaStages * (BM + BR) * kDmaBK * 2;
     static_assert(kDmaLds <= 160 * 1024, "LDS ring exceeds 160 KiB");
-    if constexpr (TM == 4 && TN == 4 && (EPI == kEpiSwiglu || EPI == kEpiPlain || EPI == kEpiResidual)) {
+    if constexpr (TM == 4 && TN == 4) {
       // the 256 x 256 block tile on 8 waves of 128 x 64, two per SIMD: one wave's barrier and load waits are the other's
       // issue slots (gate/up projection at 4096 x 4096 x 1024: 66.7 against 69.1 us), at 6 fragment reads per 8 MFMAs
       auto kern8 = gemm_nt_dma_kernel<DT, 4, 2, EPI, kDmaBK, kDmaStages, 8>;
       if (hipError_t e = DmaKernelLds<DT, 4, 2, EPI, kDmaBK, kDmaStages, 8>::entry.ensure(); e != hipSuccess) return e;
       hipLaunchKernelGGL(kern8, dim3(blocks), dim3(512), kDmaLds, s, g);
       return hipGetLastError();
+    } else {
+      auto kern = gemm_nt_dma_kernel<DT, TM, TN, EPI, kDmaBK, kDmaStages>;
+      static_assert(kDmaLds == kDmaStages * (2 * TM * 32 + 2 * TN * 32) * kDmaBK * 2, "list entry and launch disagree");
+      if (hipError_t e = DmaKernelLds<DT, TM, TN, EPI, kDmaBK, kDmaStages>::entry.ensure(); e != hipSuccess) return e;
+      hipLaunchKernelGGL(kern, dim3(blocks), dim3(kGemmThreads), kDmaLds, s, g);
+      return hipGetLastError();
     }
-    auto kern = gemm_nt_dma_kernel<DT, TM, TN, EPI, kDmaBK, kDmaStages>;
-    static_assert(kDmaLds == kDmaStages * (2 * TM * 32 + 2 * TN * 32) * kDmaBK * 2, "list entry and launch disagree");
-    if (hipError_t e = DmaKernelLds<DT, TM, TN, EPI, kDmaBK, kDmaStages>::entry.ensure(); e != hipSuccess) return e;
-    hipLaunchKernelGGL(kern, dim3(blocks), dim3(kGemmThreads), kDmaLds, s, g);
-    return hipGetLastError();
   }
   auto kern = gemm_nt_kernel<DT, TM, TN, EPI>;       // any K % 8 == 0: staged through registers
   if (hipError_t e = StagedKernelLds<DT, TM, TN, EPI>::entry.ensure(); e != hipSuccess) return e;
