@@ -5,9 +5,10 @@
  * (a hipStream_t passed as void*, NULL = the default stream) and returns without
  * waiting for the device.  The library allocates no memory: outputs and workspaces
  * come from the caller (the *_workspace_bytes calls give the sizes).  Inputs are
- * never written.  Its only global state is a per-kernel note of the devices whose
- * shared-memory limit has been raised (atomic), so calls are re-entrant as long as
- * their outputs and workspaces are distinct.
+ * never written.  Its global state is set-up that is done once per device: a per-kernel
+ * note of the devices whose shared-memory limit has been raised (atomic) and the device
+ * address of the scratch array of omni_schedule_noalloc.  Calls are re-entrant as long as
+ * their outputs and workspaces are distinct (omni_schedule_noalloc: see there).
  *
  * Return value: OMNI_OK (0); a negative OMNI_ERR_* for a rejected argument (nothing
  * was enqueued); OMNI_ERR_HIP_BASE + hipError_t when the HIP runtime refused a launch.
@@ -89,7 +90,8 @@ OMNI_API int32_t omni_router_select(const void* logits_x, const void* logits_y, 
  *                      torch.sort, :71, leaves that order open); pairs whose id is
  *                      outside [0, N) follow at positions >= offsets[N]
  *   sorted_token_ids : device [num_tokens*k] int32 (= sorted_pair_ids / k), may be NULL
- *   workspace        : device, omni_schedule_workspace_bytes() bytes */
+ *   workspace        : device, omni_schedule_workspace_bytes() bytes
+ * At most 2^30 - 1 pairs (else OMNI_ERR_SHAPE). */
 OMNI_API size_t omni_schedule_workspace_bytes(int64_t num_tokens, int32_t num_experts_per_token, int64_t num_experts);
 OMNI_API int32_t omni_schedule(const int32_t* indices, int32_t* offsets, int32_t* sorted_pair_ids,
                       int32_t* sorted_token_ids, int64_t num_tokens, int32_t num_experts_per_token,
@@ -127,7 +129,12 @@ OMNI_API int32_t omni_schedule_noalloc(const int32_t* indices, int32_t* offsets,
  *               DENSE is for the regime of the reference's group path (omni_scheduler.py:58,103-226,
  *               omni_expert.py:171-372: T*k/N > 256): a gate matrix G[T,N], C = silu(x U^T) * G on the matrix
  *               cores (kept with 16 significant bits), y = C V on the matrix cores; bf16/f16, N % 32 == 0,
- *               N <= 2048, H % 64 == 0.  AUTO takes it under the reference's rule where N <= 16 k.
+ *               N <= 2048, H % 64 == 0.  AUTO never takes it, for two differences from every other algorithm
+ *               and from the reference: it multiplies each token by EVERY table row, so a non-finite value
+ *               in a row that no token selected reaches all tokens (0 * Inf = NaN in the second GEMM), and
+ *               with f16 storage a coefficient silu(s) * g beyond 65504 becomes Inf where the others keep
+ *               it in fp32.  Where it wins (T*k/N > 256 and N <= 16 * num_experts_per_token) it wins
+ *               little; ask for it by name on finite tables.
  *   workspace : omni_expert_workspace_bytes() bytes for the same arguments (0 = may be NULL) */
 OMNI_API size_t omni_expert_workspace_bytes(int64_t num_tokens, int32_t hidden_size, int64_t num_experts,
                                    int32_t num_experts_per_token, int32_t dtype, int32_t algo);
@@ -263,6 +270,9 @@ OMNI_API int32_t omni_linear2_fwd(const void* x, const void* weight_lo, const vo
  *     average with factor 1 / num_batches_tracked (the counters are then required); one token in
  *     training is OMNI_ERR_SHAPE (nn.BatchNorm1d raises).  training == 0: the buffers
  *     normalise, nothing is written.
+ *   Limits (OMNI_ERR_UNSUPPORTED, nothing enqueued): num_expert_sqrt > 1024; and training with
+ *     momentum < 0 and k == 0 (no selection follows the statistics, and the cumulative average's
+ *     counter is advanced by the selection kernel).
  *   gates [T,k] dtype = exp(score); indices [T,k] int32; scores [T,k] dtype or NULL
  *   workspace: omni_router_workspace_bytes() bytes */
 OMNI_API size_t omni_router_workspace_bytes(int64_t num_tokens, int32_t num_expert_sqrt, int32_t dtype);

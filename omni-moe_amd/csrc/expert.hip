@@ -528,10 +528,10 @@ static int expert_dense_dispatch(const void* x, const void* up, const void* down
 // are enough pairs to amortise its second launch; otherwise rows are gathered whole.
 static int resolve_algo(int algo, int64_t T, int H, int64_t N, int k, int dtype) {
   if (algo != OMNI_EXPERT_ALGO_AUTO) return algo;
-  // the reference's rule for its group path (omni_scheduler.py:58, group_size 16): more than 256 pairs per expert --
-  // and no more than 16 experts per slot: the GEMMs cost N rows per token, the gather 2k (measured at 16384 tokens,
-  // hidden 1024: 66 us dense against 69 us gather at N = 256, k = 16; 95 against 70 at N = 512)
-  if (dense_covers(T, H, N, k, dtype) && T * (int64_t)k > 256 * N && N <= 16 * (int64_t)k) return OMNI_EXPERT_ALGO_DENSE;
+  // The dense algorithm is never chosen here: it multiplies every token by every table row, so one non-finite value
+  // in a row that nobody selected would reach every token (0 * Inf), where the other algorithms and the reference
+  // only ever touch selected rows; and where it wins at all it wins little (the reference's group regime, T*k/N > 256
+  // with N <= 16 k: 63 us against 67.5 us gather at 16384 tokens, hidden 1024, N = 256, k = 16; 95 against 70 at N = 512).
   const int es = dtype == OMNI_F32 ? 4 : 2;
   const int64_t tables = 2 * N * (int64_t)H * es;
   const bool fits = split_lanes_per_row(H, es) != 0 && k <= 2 * kWave;

@@ -19,13 +19,6 @@
 
 namespace omni {
 
-#ifdef OMNI_GEMM_TIMING
-__device__ long long* g_timing = nullptr;   // [blocks][8] cycle stamps, debug builds only
-#define OMNI_STAMP(slot) do { if (g_timing && threadIdx.x == 0) { g_timing[blockIdx.x * 8 + (slot)] = (long long)__builtin_readcyclecounter(); g_timing[blockIdx.x * 8 + 4 + (slot)] = (long long)wall_clock64(); } } while (0)
-#else
-#define OMNI_STAMP(slot) do { } while (0)
-#endif
-
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
@@ -219,7 +212,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, f32x16_t (&acc)
                 float hv[4], lv[4];
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
-                  const float c = silu_f32(acc[i][j][q4 * 4 + q]) * gt[q];
+                  const float c = gt[q] != 0.f ? silu_f32(acc[i][j][q4 * 4 + q]) * gt[q] : 0.f;   // an unselected pair contributes exactly 0, whatever its product is
                   hv[q] = Elem<DT>::round(c);
                   lv[q] = c - hv[q];
                 }
@@ -600,7 +593,6 @@ __global__ __launch_bounds__(NW * 64, 1) void gemm_nt_dma_kernel(const GemmArgs 
   };
 
   const int num_kt = g.K / BK;
-  OMNI_STAMP(0);
 #pragma unroll
   for (int t = 0; t < NS; ++t)
     if (t < num_kt) issue_tile(t);
@@ -612,7 +604,6 @@ __global__ __launch_bounds__(NW * 64, 1) void gemm_nt_dma_kernel(const GemmArgs 
   };
   wait_tile(min(NS, num_kt) - 1 < NS - 2 ? min(NS, num_kt) - 1 : NS - 2);
   __builtin_amdgcn_s_barrier();
-  OMNI_STAMP(1);
 #pragma unroll
   for (int f = 0; f < kReads; ++f) read_one(0, 0, f);
   int fetch = -1;                             // tile whose loads are half issued
@@ -632,9 +623,7 @@ __global__ __launch_bounds__(NW * 64, 1) void gemm_nt_dma_kernel(const GemmArgs 
   middle_slabs(num_kt - 1);
 #pragma unroll
   for (int ij = 0; ij < kMf; ++ij) acc[ij / TN][ij % TN] = mfma32<DT>(bf[(S - 1) & 1][ij % TN], af[(S - 1) & 1][ij / TN], acc[ij / TN][ij % TN]);
-  OMNI_STAMP(2);
   gemm_epilogue<DT, TM, TN, EPI>(g, acc, m0, n0, wm, wn, lane);
-  OMNI_STAMP(3);
 }
 
 // One list entry per kernel instantiation that launch_gemm can start (the static members come into being
@@ -875,12 +864,6 @@ extern "C" OMNI_API int32_t omni_linear2_fwd(const void* x, const void* weight_l
     default: return OMNI_ERR_DTYPE;
   }
 }
-
-#ifdef OMNI_GEMM_TIMING
-extern "C" OMNI_API int32_t omni_debug_set_timing(long long* buf) {
-  return (int32_t)hipMemcpyToSymbol(HIP_SYMBOL(omni::g_timing), &buf, sizeof(buf));
-}
-#endif
 
 namespace omni {
 // y[i] = round(y[i] + e[i]), 8 (16-bit) or 4 (fp32) elements per lane

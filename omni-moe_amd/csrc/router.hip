@@ -198,6 +198,7 @@ __device__ __forceinline__ void store_score(void* p, int64_t i, float v, int dt)
 }
 
 constexpr int kRouterWaves = 4;
+constexpr int kMaxKeys = 1024;        // keys per half that the select kernels hold (16 per lane)
 constexpr float kNegInf = -__builtin_huge_valf();
 
 struct SelectArgs {
@@ -206,6 +207,11 @@ struct SelectArgs {
   int64_t row_stride;
   const float* stats;    // NULL, or [4][r] fp32: mean_x, rstd_x, mean_y, rstd_y -> the inputs are raw
                          // projections; normalise and log-softmax them before selecting
+  const void* run_mean[2];  // instead of stats (eval-mode BatchNorm): the two halves' running_mean / running_var
+  const void* run_var[2];   //   [r] of dtype stat_dt; mean and 1/sqrt(var + eps) are formed here, and block 0
+  float* stats_out;         //   also leaves them at stats_out [4][r] (may be NULL) for a backward pass
+  int stat_dt;
+  float eps;
   void* scores;          // [T,k] storage dtype, may be NULL
   void* gates;           // [T,k] storage dtype = exp(score), may be NULL
   int32_t* indices;      // [T,k]
@@ -220,18 +226,35 @@ __device__ __forceinline__ void count_batch(const SelectArgs& g) {
     if (g.count_batch[0]) *g.count_batch[0] += 1;
     if (g.count_batch[1]) *g.count_batch[1] += 1;
   }
+  if (blockIdx.x == 0 && !g.stats && g.run_mean[0] && g.stats_out) {   // eval mode: the statistics a backward pass reads
+    for (int i = threadIdx.x; i < 2 * g.r; i += blockDim.x) {
+      const int half = i >= g.r, key = i - half * g.r;
+      g.stats_out[(2 * half) * g.r + key] = load_score(g.run_mean[half], key, g.stat_dt);
+      g.stats_out[(2 * half + 1) * g.r + key] = 1.0f / sqrtf(load_score(g.run_var[half], key, g.stat_dt) + g.eps);
+    }
+  }
 }
 
 // BatchNorm (affine-free) then log-softmax of one half, in place: v holds the raw projection
 // of key a*64+lane (NaN-free -inf padding past r).  Each stage rounds to the storage dtype
 // where the reference's torch ops do (BN output, log-softmax output; omni_moe.py:70-78).
 template <int R>
-__device__ __forceinline__ void normalise_half(float (&v)[R], const float* mean, const float* rstd, int r, int lane, int dt) {
+__device__ __forceinline__ void normalise_half(float (&v)[R], const SelectArgs& g, const int half, int r, int lane, int dt) {
   float m = kNegInf;
 #pragma unroll
   for (int a = 0; a < R; ++a) {
     const int key = a * kWave + lane;
-    if (key < r) v[a] = round_score((v[a] - mean[key]) * rstd[key], dt);
+    if (key < r) {
+      float mean, rstd;
+      if (g.stats) {
+        mean = g.stats[(2 * half) * r + key];
+        rstd = g.stats[(2 * half + 1) * r + key];
+      } else {                                   // the same expressions as bn_finalize_kernel's
+        mean = load_score(g.run_mean[half], key, g.stat_dt);
+        rstd = 1.0f / sqrtf(load_score(g.run_var[half], key, g.stat_dt) + g.eps);
+      }
+      v[a] = round_score((v[a] - mean) * rstd, dt);
+    }
     m = fmaxf(m, v[a]);
   }
   m = wave_max(m);
@@ -279,9 +302,9 @@ __global__ __launch_bounds__(kRouterWaves* kWave) void router_select_kernel(cons
       sy[a] = ok ? load_score(g.ly, int64_t(t) * g.row_stride + key, dt) : kNegInf;
       px[a] = py[a] = key;
     }
-    if (g.stats) {
-      normalise_half<R>(sx, g.stats, g.stats + r, r, lane, dt);
-      normalise_half<R>(sy, g.stats + 2 * r, g.stats + 3 * r, r, lane, dt);
+    if (g.stats || g.run_mean[0]) {
+      normalise_half<R>(sx, g, 0, r, lane, dt);
+      normalise_half<R>(sy, g, 1, r, lane, dt);
     }
     bitonic_sort2<R>(sx, px, sy, py, lane);
 
@@ -439,9 +462,9 @@ __global__ __launch_bounds__(kRouterWaves* kWave) void router_select_packed_kern
       sx[a] = ok ? load_score(g.lx, int64_t(t) * g.row_stride + key, dt) : kNegInf;
       sy[a] = ok ? load_score(g.ly, int64_t(t) * g.row_stride + key, dt) : kNegInf;
     }
-    if (g.stats) {
-      normalise_half<R>(sx, g.stats, g.stats + r, r, lane, dt);
-      normalise_half<R>(sy, g.stats + 2 * r, g.stats + 3 * r, r, lane, dt);
+    if (g.stats || g.run_mean[0]) {
+      normalise_half<R>(sx, g, 0, r, lane, dt);
+      normalise_half<R>(sy, g, 1, r, lane, dt);
     }
     uint32_t kx[R], ky[R];
 #pragma unroll
@@ -517,7 +540,7 @@ static int select_dispatch(SelectArgs g, hipStream_t s) {
   else if (rpl <= 4) err = select_by_cells<4>(cpl, g, s);
   else if (rpl <= 8) err = select_by_cells<8>(cpl, g, s);
   else if (rpl <= 16) err = select_by_cells<16>(cpl, g, s);
-  else return OMNI_ERR_UNSUPPORTED;                          // r > 1024
+  else return OMNI_ERR_UNSUPPORTED;                          // r > kMaxKeys: the entry points refuse it before anything is enqueued
   return err == hipSuccess ? OMNI_OK : OMNI_ERR_HIP_BASE + (int)err;
 }
 
@@ -600,7 +623,10 @@ extern "C" OMNI_API int32_t omni_router_select(const void* logits_x, const void*
   if (dtype != OMNI_BF16 && dtype != OMNI_F16 && dtype != OMNI_F32) return OMNI_ERR_DTYPE;
   if (num_tokens == 0 || k == 0) return OMNI_OK;
   if (!logits_x || !logits_y || !scores || !indices) return OMNI_ERR_NULL;
-  SelectArgs g{logits_x, logits_y, r, nullptr, scores, nullptr, indices, (int)num_tokens, r, k, 0, dtype, {}, {nullptr, nullptr}};
+  if (r > kMaxKeys) return OMNI_ERR_UNSUPPORTED;
+  SelectArgs g{};
+  g.lx = logits_x; g.ly = logits_y; g.row_stride = r; g.scores = scores; g.indices = indices;
+  g.num_tokens = (int)num_tokens; g.r = r; g.k = k; g.dt = dtype;
   return select_dispatch(g, (hipStream_t)stream);
 }
 
@@ -640,6 +666,7 @@ extern "C" OMNI_API int32_t omni_router_fwd(const void* x, const void* weight_x,
   if (!x || !weight_x || !weight_y || !running_mean_x || !running_var_x || !running_mean_y || !running_var_y) return OMNI_ERR_NULL;
   if (training && momentum < 0.f && (!num_batches_tracked_x || !num_batches_tracked_y)) return OMNI_ERR_NULL;   // the cumulative average needs the counts
   if (training && momentum < 0.f && k == 0) return OMNI_ERR_UNSUPPORTED;
+  if (r > kMaxKeys) return OMNI_ERR_UNSUPPORTED;           // the select kernels' limit, checked before the projection is enqueued
   if (k > 0 && (!gates || !indices)) return OMNI_ERR_NULL;
   if (!workspace) return OMNI_ERR_WORKSPACE;
   hipStream_t s = (hipStream_t)stream;
@@ -655,14 +682,28 @@ extern "C" OMNI_API int32_t omni_router_fwd(const void* x, const void* weight_x,
   // (in training its epilogue also leaves the per-32-row column statistics)
   if (int e = omni_gemm_router_projection(x, weight_x, weight_y, z, training ? part_mean : nullptr, training ? part_m2 : nullptr,
                                           num_tokens, hidden_size, r, dtype, stream)) return e;
-  BnFinalArgs b{part_mean, part_m2, stats, {running_mean_x, running_mean_y}, {running_var_x, running_var_y},
-                {num_batches_tracked_x, num_batches_tracked_y}, (int)num_tokens, r, (int)strips, training ? 1 : 0, stats_dtype,
-                k == 0 ? 1 : 0, momentum, eps};
-  hipLaunchKernelGGL(bn_finalize_kernel, dim3((2 * r + 3) / 4), dim3(256), 0, s, b);
-  hipError_t err = hipGetLastError();
-  if (err != hipSuccess) return OMNI_ERR_HIP_BASE + (int)err;
-  if (k == 0) return OMNI_OK;
-  SelectArgs g{z, (const char*)z + (size_t)r * es, 2 * r, stats, scores, gates, indices, (int)num_tokens, r, k, 0, dtype, {},
-               {training ? num_batches_tracked_x : nullptr, training ? num_batches_tracked_y : nullptr}};
+  // Training: one more launch merges the partial statistics and moves the running buffers.  In eval mode the
+  // select kernel reads the running buffers itself (and leaves mean and 1/sqrt(var + eps) in `stats`).
+  if (training || k == 0) {
+    BnFinalArgs b{part_mean, part_m2, stats, {running_mean_x, running_mean_y}, {running_var_x, running_var_y},
+                  {num_batches_tracked_x, num_batches_tracked_y}, (int)num_tokens, r, (int)strips, training ? 1 : 0, stats_dtype,
+                  k == 0 ? 1 : 0, momentum, eps};
+    hipLaunchKernelGGL(bn_finalize_kernel, dim3((2 * r + 3) / 4), dim3(256), 0, s, b);
+    hipError_t err = hipGetLastError();
+    if (err != hipSuccess) return OMNI_ERR_HIP_BASE + (int)err;
+    if (k == 0) return OMNI_OK;
+  }
+  SelectArgs g{};
+  g.lx = z; g.ly = (const char*)z + (size_t)r * es; g.row_stride = 2 * r;
+  g.scores = scores; g.gates = gates; g.indices = indices;
+  g.num_tokens = (int)num_tokens; g.r = r; g.k = k; g.dt = dtype;
+  if (training) {
+    g.stats = stats;
+    g.count_batch[0] = num_batches_tracked_x; g.count_batch[1] = num_batches_tracked_y;
+  } else {
+    g.run_mean[0] = running_mean_x; g.run_mean[1] = running_mean_y;
+    g.run_var[0] = running_var_x; g.run_var[1] = running_var_y;
+    g.stats_out = stats; g.stat_dt = stats_dtype; g.eps = eps;
+  }
   return select_dispatch(g, s);
 }

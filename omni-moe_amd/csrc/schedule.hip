@@ -58,7 +58,9 @@ struct SortPass {
   uint32_t mask;            //   ... & mask (0xFFFFFFFF on the last pass)
   int last;                 // last pass: ids outside [0, N) go to bin bins-1; earlier passes: to bin 0
   uint32_t num_experts;
-  uint64_t inv_top_k;       // ceil(2^40 / top_k): (v * inv_top_k) >> 40 == v / top_k for every v < 2^31 and top_k <= 2^9
+  uint64_t inv_top_k;       // ceil(2^s / top_k) with s = inv_shift = 30 + ceil(log2(top_k)): (v * inv_top_k) >> s == v / top_k for
+  int inv_shift;            // every pair id v < 2^30 (the excess v * (inv_top_k * top_k - 2^s) / (top_k * 2^s) stays below
+                            // 1 / top_k, and the product below 2^62)
 };
 
 __device__ __forceinline__ int sort_digit(const SortPass& a, int32_t key) {
@@ -269,7 +271,7 @@ __global__ __launch_bounds__(kSortThreads) void sort_scatter_kernel(const SortPa
       if (active) {
         if (a.keys_out) a.keys_out[pos[u]] = keys[u];
         a.vals_out[pos[u]] = vals[u];
-        if (a.tok_out) a.tok_out[pos[u]] = (int32_t)(((uint64_t)(uint32_t)vals[u] * a.inv_top_k) >> 40);   // val / top_k
+        if (a.tok_out) a.tok_out[pos[u]] = (int32_t)(((uint64_t)(uint32_t)vals[u] * a.inv_top_k) >> a.inv_shift);   // val / top_k
       }
     }
   }
@@ -375,7 +377,9 @@ extern "C" OMNI_API int32_t omni_schedule(const int32_t* indices, int32_t* offse
       a.mask = (pl.passes == 2 && pass == 0) ? (uint32_t)((1 << pl.lo_bits) - 1) : 0xFFFFFFFFu;
       a.last = last ? 1 : 0;
       a.num_experts = (uint32_t)N;
-      a.inv_top_k = num_experts_per_token > 0 ? ((1ull << 40) + num_experts_per_token - 1) / (uint64_t)num_experts_per_token : 0;
+      a.inv_shift = 30;
+      while ((1ll << (a.inv_shift - 30)) < (int64_t)num_experts_per_token) ++a.inv_shift;
+      a.inv_top_k = num_experts_per_token > 0 ? ((1ull << a.inv_shift) + num_experts_per_token - 1) / (uint64_t)num_experts_per_token : 0;
       hipLaunchKernelGGL(sort_count_kernel, dim3(a.tiles), dim3(kSortThreads), (size_t)a.stride * 4, s, a);
       hipLaunchKernelGGL(sort_scatter_kernel, dim3(a.tiles * kSlices), dim3(kSortThreads), 0, s, a);
     }

@@ -13,11 +13,15 @@ stage -- Linear, BatchNorm1d, log_softmax, router op, exp -- as one node, the ex
 MLP op, add), so the layer trains; call it under ``torch.no_grad()`` for the fused path.
 """
 import math
+import threading
 
 import torch
 import torch.nn as nn
 
 from omni_moe.ops.hip import hip_omni_expert_func, hip_omni_mlp_func, hip_omni_moe_fwd_func, hip_omni_router_fwd_func
+
+
+_BRANCH_RESOURCES = {}      # (device index, host thread) -> (side stream, fork event, join event)
 
 
 class OmniMoEConfig:
@@ -95,16 +99,21 @@ class OmniMoE(nn.Module):
     # intermediate; 2048 x 1024 x 4096 measured level on an MI355X) the call would be host-bound: one stream then.
     overlap_min_work = 2 ** 33
 
-    def _branch_resources(self, device):
-        res = self.__dict__.get("_omni_branch")
-        if res is None or res[0].device != device:
+    @staticmethod
+    def _branch_resources(device):
+        """Side stream and the fork / join events for ``device``, one set per device and host thread.  They live in a
+        table of this module, not on the layer: a layer stays a plain ``nn.Module`` that ``copy.deepcopy``,
+        ``torch.save`` and ``state_dict`` treat as the reference's, and layers that run one after another on a
+        stream share the set (an event is recorded and waited for again by every call)."""
+        key = (device.index if device.index is not None else torch.cuda.current_device(), threading.get_ident())
+        res = _BRANCH_RESOURCES.get(key)
+        if res is None:
             with torch.cuda.device(device):
                 side = torch.cuda.Stream(device=device)
                 fork, join = torch.cuda.Event(), torch.cuda.Event()
                 fork.record()                                # events come into being when first recorded
                 join.record()
-            res = (side, fork, join)
-            self.__dict__["_omni_branch"] = res
+            res = _BRANCH_RESOURCES[key] = (side, fork, join)
         return res
 
     def _forward_differentiable(self, hidden_states: torch.Tensor) -> torch.Tensor:

@@ -583,8 +583,8 @@ def hip_omni_moe_fwd_func(
     T, H = x.shape
     I, N, r, k = gate_weight.size(0), up_embed.size(0), router_weight_x.size(0), int(num_experts_per_token)
     weights = (gate_weight, up_weight, down_weight, router_weight_x, router_weight_y, up_embed, down_embed)
-    if x.dim() != 2 or x.dtype not in _lib.DTYPE_CODE or any(t.dtype != x.dtype or not t.is_contiguous() for t in weights):
-        raise TypeError("x and the weights must be contiguous and share a dtype in {bfloat16, float16, float32}")
+    if x.dim() != 2 or x.dtype not in _lib.DTYPE_CODE or any(t.dtype != x.dtype for t in weights):
+        raise TypeError("x and the weights must share a dtype in {bfloat16, float16, float32}")
     if (gate_weight.shape != (I, H) or up_weight.shape != (I, H) or down_weight.shape != (H, I) or router_weight_y.shape != (r, H)
             or router_weight_x.shape != (r, H) or up_embed.shape != (N, H) or down_embed.shape != (N, H)):
         raise ValueError("weight shapes do not fit (tokens, hidden) input")
@@ -598,6 +598,8 @@ def hip_omni_moe_fwd_func(
     momentum = -1.0 if momentum is None else momentum
     dev = _lib.require_gpu(x, *weights, *stats)
     x = _c(x)
+    # the reference makes every tensor argument of its operators contiguous (utils.py:47-65)
+    gate_weight, up_weight, down_weight, router_weight_x, router_weight_y, up_embed, down_embed = (_c(t) for t in weights)
     lib = _lib.load()
     dt = _lib.DTYPE_CODE[x.dtype]
     y = torch.empty_like(x)

@@ -1,13 +1,17 @@
-/* A plain C caller that runs one compute entry of libomni_moe_hip.so on the GPU: omni_router_select on device buffers
+/* A plain C caller that runs compute entries of libomni_moe_hip.so on the GPU: omni_router_select on device buffers
  * it allocates and fills through the HIP runtime's C API, checked against a scalar loop over the same inputs; then
- * omni_init() followed by a HIP-graph capture of omni_schedule for a shape that never ran eagerly (its kernel needs
- * more than the default dynamic LDS, which omni_init has already arranged), replayed and checked the same way.
+ * omni_init(), and straight after it -- no eager call came before -- HIP-graph captures of
+ *   - omni_linear_fwd at a shape whose kernel needs 128 KiB of dynamic LDS: without omni_init() the call would have
+ *     to raise that kernel's limit with hipFuncSetAttribute inside the capture; omni_init() has done it for every kernel,
+ *   - omni_schedule and omni_schedule_noalloc side by side (the second on the device scratch that omni_init() resolved),
+ * each replayed three times and checked against scalar loops.
  * Built (gcc) and run by tests/test_gpu_c_client.py on the GPU box. */
 #define __HIP_PLATFORM_AMD__ 1
 #include <hip/hip_runtime_api.h>
 #include <stdint.h>
 #include <stdio.h>
 #include <stdlib.h>
+#include <string.h>
 
 #include "omni_moe_hip.h"
 
@@ -16,45 +20,93 @@
 enum { T = 37, R = 8, K = 6 };
 enum { ST = 300, SK = 4, SN = 4096, SP = ST * SK };
 
-/* omni_schedule inside a stream capture, straight after omni_init(): no eager call of this shape came before */
+enum { GM = 2048, GN = 2048, GK = 64 };
+
+/* bf16 bits of a small integer (exactly representable) and back */
+static uint16_t bf16_of_int(int v) { float f = (float)v; uint32_t u; memcpy(&u, &f, 4); return (uint16_t)(u >> 16); }
+static float float_of_bf16(uint16_t b) { uint32_t u = (uint32_t)b << 16; float f; memcpy(&f, &u, 4); return f; }
+
+/* omni_linear_fwd inside a stream capture, straight after omni_init().  2048 x 2048 outputs make the library pick its
+ * 128 x 128 tile, whose kernel needs 128 KiB of dynamic LDS.  Operands are small integers, so every product and sum is
+ * exact and the result must equal the scalar loop bit for bit. */
+static int captured_gemm(void) {
+  uint16_t* x = (uint16_t*)malloc((size_t)GM * GK * 2); uint16_t* w = (uint16_t*)malloc((size_t)GN * GK * 2);
+  uint16_t* y = (uint16_t*)malloc((size_t)GM * GN * 2);
+  int8_t* xi = (int8_t*)malloc((size_t)GM * GK); int8_t* wi = (int8_t*)malloc((size_t)GN * GK);
+  if (!x || !w || !y || !xi || !wi) return 30;
+  uint32_t s = 4242u;
+  for (int i = 0; i < GM * GK; ++i) { s = s * 1664525u + 1013904223u; xi[i] = (int8_t)((int)((s >> 12) % 5) - 2); x[i] = bf16_of_int(xi[i]); }
+  for (int i = 0; i < GN * GK; ++i) { s = s * 1664525u + 1013904223u; wi[i] = (int8_t)((int)((s >> 12) % 3) - 1); w[i] = bf16_of_int(wi[i]); }
+  void *dx, *dw, *dy;
+  CHECK(hipMalloc(&dx, (size_t)GM * GK * 2)); CHECK(hipMalloc(&dw, (size_t)GN * GK * 2)); CHECK(hipMalloc(&dy, (size_t)GM * GN * 2));
+  CHECK(hipMemcpy(dx, x, (size_t)GM * GK * 2, hipMemcpyHostToDevice)); CHECK(hipMemcpy(dw, w, (size_t)GN * GK * 2, hipMemcpyHostToDevice));
+  hipStream_t stream; hipGraph_t graph; hipGraphExec_t exec;
+  CHECK(hipStreamCreate(&stream));
+  CHECK(hipStreamBeginCapture(stream, hipStreamCaptureModeGlobal));
+  const int32_t code = omni_linear_fwd(dx, dw, NULL, dy, GM, GK, GN, OMNI_BF16, stream);
+  const hipError_t end = hipStreamEndCapture(stream, &graph);
+  if (code != OMNI_OK) { printf("omni_linear_fwd under capture: %s\n", omni_error_string(code)); return 31; }
+  CHECK(end);
+  CHECK(hipGraphInstantiate(&exec, graph, NULL, NULL, 0));
+  for (int rep = 0; rep < 3; ++rep) {
+    CHECK(hipMemset(dy, 0xff, (size_t)GM * GN * 2));
+    CHECK(hipGraphLaunch(exec, stream));
+    CHECK(hipStreamSynchronize(stream));
+    CHECK(hipMemcpy(y, dy, (size_t)GM * GN * 2, hipMemcpyDeviceToHost));
+    for (int m = 0; m < GM; ++m)
+      for (int n = 0; n < GN; ++n) {
+        int acc = 0;
+        for (int k = 0; k < GK; ++k) acc += xi[m * GK + k] * wi[n * GK + k];      /* |acc| <= 128: exact in bf16 */
+        if (float_of_bf16(y[(size_t)m * GN + n]) != (float)acc) { printf("gemm replay %d: y[%d][%d] = %g, want %d\n", rep, m, n, float_of_bf16(y[(size_t)m * GN + n]), acc); return 32; }
+      }
+  }
+  CHECK(hipGraphExecDestroy(exec)); CHECK(hipGraphDestroy(graph)); CHECK(hipStreamDestroy(stream));
+  CHECK(hipFree(dx)); CHECK(hipFree(dw)); CHECK(hipFree(dy));
+  free(x); free(w); free(y); free(xi); free(wi);
+  return 0;
+}
+
+/* omni_schedule and omni_schedule_noalloc inside one stream capture: no eager call of this shape came before */
 static int captured_schedule(void) {
   static int32_t ids[SP], offsets[SN + 1], pairs[SP], tokens[SP], want_off[SN + 1], fill[SN];
   uint32_t s = 777u;
   for (int i = 0; i < SP; ++i) { s = s * 1664525u + 1013904223u; ids[i] = (int32_t)((s >> 10) % SN); }
-  int32_t code = omni_init();
-  if (code != OMNI_OK) { printf("omni_init: %s\n", omni_error_string(code)); return 20; }
-  if (omni_init() != OMNI_OK) { printf("second omni_init failed\n"); return 21; }
   const size_t ws_bytes = omni_schedule_workspace_bytes(ST, SK, SN);
-  void *dids, *doff, *dpairs, *dtok, *dws;
-  CHECK(hipMalloc(&dids, sizeof ids)); CHECK(hipMalloc(&doff, sizeof offsets)); CHECK(hipMalloc(&dpairs, sizeof pairs));
-  CHECK(hipMalloc(&dtok, sizeof tokens)); CHECK(hipMalloc(&dws, ws_bytes));
+  void *dids, *doff[2], *dpairs[2], *dtok[2], *dws;
+  CHECK(hipMalloc(&dids, sizeof ids)); CHECK(hipMalloc(&dws, ws_bytes));
+  for (int v = 0; v < 2; ++v) { CHECK(hipMalloc(&doff[v], sizeof offsets)); CHECK(hipMalloc(&dpairs[v], sizeof pairs)); CHECK(hipMalloc(&dtok[v], sizeof tokens)); }
   CHECK(hipMemcpy(dids, ids, sizeof ids, hipMemcpyHostToDevice));
   hipStream_t stream; hipGraph_t graph; hipGraphExec_t exec;
   CHECK(hipStreamCreate(&stream));
   CHECK(hipStreamBeginCapture(stream, hipStreamCaptureModeGlobal));
-  code = omni_schedule((const int32_t*)dids, (int32_t*)doff, (int32_t*)dpairs, (int32_t*)dtok, ST, SK, SN, dws, stream);
+  const int32_t code = omni_schedule((const int32_t*)dids, (int32_t*)doff[0], (int32_t*)dpairs[0], (int32_t*)dtok[0], ST, SK, SN, dws, stream);
+  const int32_t code2 = omni_schedule_noalloc((const int32_t*)dids, (int32_t*)doff[1], (int32_t*)dpairs[1], (int32_t*)dtok[1], ST, SK, SN, stream);
   const hipError_t end = hipStreamEndCapture(stream, &graph);
   if (code != OMNI_OK) { printf("omni_schedule under capture: %s\n", omni_error_string(code)); return 22; }
+  if (code2 != OMNI_OK) { printf("omni_schedule_noalloc under capture: %s\n", omni_error_string(code2)); return 25; }
   CHECK(end);
   CHECK(hipGraphInstantiate(&exec, graph, NULL, NULL, 0));
   for (int i = 0; i <= SN; ++i) want_off[i] = 0;
   for (int i = 0; i < SP; ++i) want_off[ids[i] + 1]++;
   for (int i = 0; i < SN; ++i) want_off[i + 1] += want_off[i];
   for (int rep = 0; rep < 3; ++rep) {
-    CHECK(hipMemset(doff, 0xff, sizeof offsets)); CHECK(hipMemset(dpairs, 0xff, sizeof pairs)); CHECK(hipMemset(dtok, 0xff, sizeof tokens));
+    for (int v = 0; v < 2; ++v) { CHECK(hipMemset(doff[v], 0xff, sizeof offsets)); CHECK(hipMemset(dpairs[v], 0xff, sizeof pairs)); CHECK(hipMemset(dtok[v], 0xff, sizeof tokens)); }
     CHECK(hipGraphLaunch(exec, stream));
     CHECK(hipStreamSynchronize(stream));
-    CHECK(hipMemcpy(offsets, doff, sizeof offsets, hipMemcpyDeviceToHost)); CHECK(hipMemcpy(pairs, dpairs, sizeof pairs, hipMemcpyDeviceToHost));
-    CHECK(hipMemcpy(tokens, dtok, sizeof tokens, hipMemcpyDeviceToHost));
-    for (int i = 0; i < SN; ++i) fill[i] = 0;
-    for (int i = 0; i <= SN; ++i) if (offsets[i] != want_off[i]) { printf("replay %d: offsets[%d] = %d, want %d\n", rep, i, offsets[i], want_off[i]); return 23; }
-    for (int i = 0; i < SP; ++i) {                       /* stable: pair i lands at its expert's next free slot */
-      const int32_t slot = want_off[ids[i]] + fill[ids[i]]++;
-      if (pairs[slot] != i || tokens[slot] != i / SK) { printf("replay %d: slot %d holds pair %d token %d, want %d %d\n", rep, slot, pairs[slot], tokens[slot], i, i / SK); return 24; }
+    for (int v = 0; v < 2; ++v) {
+      CHECK(hipMemcpy(offsets, doff[v], sizeof offsets, hipMemcpyDeviceToHost)); CHECK(hipMemcpy(pairs, dpairs[v], sizeof pairs, hipMemcpyDeviceToHost));
+      CHECK(hipMemcpy(tokens, dtok[v], sizeof tokens, hipMemcpyDeviceToHost));
+      for (int i = 0; i < SN; ++i) fill[i] = 0;
+      for (int i = 0; i <= SN; ++i) if (offsets[i] != want_off[i]) { printf("replay %d entry %d: offsets[%d] = %d, want %d\n", rep, v, i, offsets[i], want_off[i]); return 23; }
+      for (int i = 0; i < SP; ++i) {                       /* stable: pair i lands at its expert's next free slot */
+        const int32_t slot = want_off[ids[i]] + fill[ids[i]]++;
+        if (pairs[slot] != i || tokens[slot] != i / SK) { printf("replay %d entry %d: slot %d holds pair %d token %d, want %d %d\n", rep, v, slot, pairs[slot], tokens[slot], i, i / SK); return 24; }
+      }
     }
   }
   CHECK(hipGraphExecDestroy(exec)); CHECK(hipGraphDestroy(graph)); CHECK(hipStreamDestroy(stream));
-  CHECK(hipFree(dids)); CHECK(hipFree(doff)); CHECK(hipFree(dpairs)); CHECK(hipFree(dtok)); CHECK(hipFree(dws));
+  CHECK(hipFree(dids)); CHECK(hipFree(dws));
+  for (int v = 0; v < 2; ++v) { CHECK(hipFree(doff[v])); CHECK(hipFree(dpairs[v])); CHECK(hipFree(dtok[v])); }
   return 0;
 }
 
@@ -94,8 +146,13 @@ int main(void) {
     }
   }
   CHECK(hipFree(dlx)); CHECK(hipFree(dly)); CHECK(hipFree(dscores)); CHECK(hipFree(dids));
+  int32_t init = omni_init();
+  if (init != OMNI_OK) { printf("omni_init: %s\n", omni_error_string(init)); return 20; }
+  if (omni_init() != OMNI_OK) { printf("second omni_init failed\n"); return 21; }
+  const int gemm = captured_gemm();
+  if (gemm) return gemm;
   const int sched = captured_schedule();
   if (sched) return sched;
-  printf("c abi gpu ok: %d tokens routed, %d pairs scheduled from a captured graph\n", T, SP);
+  printf("c abi gpu ok: %d tokens routed, a %d x %d x %d product and %d pairs scheduled (with and without workspace) from captured graphs\n", T, GM, GN, GK, SP);
   return 0;
 }

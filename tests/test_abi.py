@@ -86,9 +86,35 @@ def test_argument_errors_need_no_gpu():
     assert lib.omni_moe_fwd(*([p] * 15), 1, 64, 64, 16, 4, 2, 0, 2, 1, 0.1, 1e-5, p, None, None, None, None) == -2
     assert lib.omni_router_fwd(*([p] * 9), 1, 0.1, 1e-5, p, p, None, 1, 64, 4, 2, 0, 2, p, None) == -2
     assert lib.omni_router_fwd(p, p, p, p, p, None, p, p, None, 1, -1.0, 1e-5, p, p, None, 4, 64, 4, 2, 0, 2, p, None) == -1   # cumulative average needs the counters
+    # limits of the select kernels and of the schedule's multiply-shift division: refused before anything is enqueued
+    assert lib.omni_router_fwd(*([p] * 9), 0, 0.1, 1e-5, p, p, None, 4, 64, 1025, 2, 0, 2, p, None) == -5      # r > 1024
+    assert lib.omni_router_select(p, p, p, p, 4, 1025, 2, 0, None) == -5
+    assert lib.omni_schedule(p, p, p, p, 1 << 20, 1024, 16, p, None) == -2                                      # 2^30 pairs
     import torch
     if not torch.cuda.is_available():
         assert lib.omni_init() >= 1000           # a HIP error (no device), not a crash
+
+
+def test_schedule_token_id_division_is_exact():
+    """The schedule writes sorted_token_ids = pair_id // top_k as (pair_id * ceil(2^s / top_k)) >> s with
+    s = 30 + ceil(log2(top_k)) (schedule.hip); the entry points admit pair ids below 2^30.  Within that bound the
+    multiply-shift must equal the integer division for every top_k, in 64-bit arithmetic.  Checked where it would
+    break first: the last pair id before each multiple of top_k and the multiple itself, near the top of the range."""
+    import numpy as np
+    top = (1 << 30) - 1
+    for k in list(range(1, 2100)) + [4095, 4096, 4097, 65535, 65537, (1 << 20) + 1, top]:
+        s = 30
+        while (1 << (s - 30)) < k:
+            s += 1
+        inv = ((1 << s) + k - 1) // k
+        assert top * inv < 1 << 64                         # the product never wraps
+        q = np.arange(max(top // k - 64, 0), top // k + 1, dtype=np.uint64)
+        v = np.concatenate([q * np.uint64(k) + np.uint64(k - 1), q * np.uint64(k), np.arange(0, min(4 * k, 8192), dtype=np.uint64)])
+        v = v[v <= top]
+        assert np.array_equal((v * np.uint64(inv)) >> np.uint64(s), v // np.uint64(k)), k
+    # a fixed shift of 40 is not enough beyond top_k = 1024 (and wraps for small top_k), which is why s follows top_k
+    k, v = 1038, 1073741453
+    assert (v * (((1 << 40) + k - 1) // k)) >> 40 != v // k
 
 
 def test_ops_fail_loudly_without_gpu():
@@ -116,6 +142,24 @@ def test_reference_import_paths():
     assert layer.num_expert_sqrt == 16 and layer.up_embed.weight.shape == (256, 64)
     with pytest.raises(ValueError):
         OmniMoE(OmniMoEConfig(64, 128, "gelu", 256, 8))
+
+
+def test_layer_is_a_plain_module_on_the_cpu(tmp_path):
+    """Nothing on a layer stands in the way of copy.deepcopy, pickling or a state_dict round trip (the
+    side stream and events of the two-stream forward live outside the module)."""
+    import copy
+    import torch
+    from omni_moe.modules.omni_moe import OmniMoE, OmniMoEConfig
+    layer = OmniMoE(OmniMoEConfig(64, 128, "silu", 256, 8))
+    twin = copy.deepcopy(layer)
+    assert all(torch.equal(a, b) for a, b in zip(layer.state_dict().values(), twin.state_dict().values()))
+    path = str(tmp_path / "layer.pt")
+    torch.save(layer, path)
+    loaded = torch.load(path, weights_only=False)           # a file this test wrote itself
+    assert sorted(loaded.state_dict()) == sorted(layer.state_dict())
+    other = OmniMoE(OmniMoEConfig(64, 128, "silu", 256, 8))
+    other.load_state_dict(layer.state_dict())
+    assert torch.equal(other.up_embed.weight, layer.up_embed.weight)
 
 
 def test_header_is_plain_c_and_a_c_program_links(tmp_path):

@@ -1,6 +1,7 @@
 """The C ABI from plain C on the GPU: tests/c_abi_gpu_client.c allocates device buffers with the HIP runtime's C API, calls
 omni_router_select through include/omni_moe_hip.h and checks ids and scores against a scalar loop; it then calls omni_init()
-and captures omni_schedule into a HIP graph without any eager call of that shape before, and checks three replays."""
+and captures, without any eager call before, a GEMM whose kernel needs 128 KiB of dynamic LDS and the two schedule entry
+points into HIP graphs, and checks three replays of each."""
 import os
 import subprocess
 

@@ -20,8 +20,9 @@ def _ops():
     return hip
 
 
-MLP_CASES = [(1024, 1024, 1024), (1024, 1024, 4096), (4096, 1024, 4096), (333, 256, 1000), (128, 64, 128),
-             (512, 2048, 8192), (5, 8, 8)]
+# the first four are the reference's benchmark grid (tests/test_mlp.py:144-150): intermediate 1024 .. 65536
+MLP_CASES = [(1024, 1024, 1024), (1024, 1024, 4096), (1024, 1024, 16384), (1024, 1024, 65536), (4096, 1024, 4096),
+             (333, 256, 1000), (128, 64, 128), (512, 2048, 8192), (5, 8, 8)]
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
@@ -273,13 +274,15 @@ def test_layer_config5_large_skewed(device):
     torch.testing.assert_close(gates.cpu()[sub].float(), want_g.float(), rtol=2e-2, atol=2e-2)
 
 
+@pytest.mark.parametrize("training", [False, True], ids=["eval", "train"])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
 @pytest.mark.parametrize("two_streams", [False, True], ids=["one-stream", "two-streams"])
-def test_layer_expert_term_visible_auto_split(two_streams, dtype, device):
+def test_layer_expert_term_visible_auto_split(two_streams, dtype, training, device):
     """A layer whose expert branch is as large as its MLP branch (weights ~ N(0, 0.1)) and whose shape makes the layer call
     pick the hidden-split expert algorithm (4096 tokens x 8 = 32768 pairs, tables that overflow one L2): y - mlp must equal
     the oracle's expert term on the expert term's own scale, on one stream and on two.  A layer that dropped or mis-wired
-    router -> experts (wrong gates or ids buffer, workspace overlap, missing join) fails here."""
+    router -> experts (wrong gates or ids buffer, workspace overlap, missing join) fails here.  In training mode the router
+    normalises with the statistics of the whole 4096-token batch, on the device and in the oracle."""
     from omni_moe.modules.omni_moe import OmniMoE, OmniMoEConfig
     T, H, I, N, k = 4096, 512, 512, (1024 if dtype == torch.float32 else 4096), 8
     x, w = oracle.make_layer_inputs(21, T, H, I, N, dtype=dtype, w_std=0.1)
@@ -289,21 +292,23 @@ def test_layer_expert_term_visible_auto_split(two_streams, dtype, device):
     layer.load_state_dict({"gate_proj.weight": w.gate_proj, "up_proj.weight": w.up_proj, "down_proj.weight": w.down_proj,
                            "router_gate_x.weight": w.router_gate_x, "router_gate_y.weight": w.router_gate_y,
                            "up_embed.weight": w.up_embed, "down_embed.weight": w.down_embed}, strict=False)
-    layer = layer.to(device=device, dtype=dtype).eval()      # eval: token-independent, the oracle needs no batch statistics
+    layer = layer.to(device=device, dtype=dtype).train(training)
     layer.overlap_branches = two_streams
     layer.overlap_min_work = 0
     from omni_moe.ops.hip import _lib
     lib = _lib.load()
     es = 4 if dtype == torch.float32 else 2
     assert lib.omni_expert_workspace_bytes(T, H, N, k, _lib.DTYPE_CODE[dtype], _lib.ALGO_AUTO) == 8 * T * k * 4, "AUTO should pick the split algorithm here"
-    print(f"layer with visible expert term, {dtype}, two_streams={two_streams}", flush=True)
+    print(f"layer with visible expert term, {dtype}, two_streams={two_streams}, training={training}", flush=True)
     xd = x.to(device)
     y = layer(xd).view(-1, H)
     mlp = _ops().hip_omni_mlp_func(xd.view(-1, H), layer.gate_proj.weight, layer.up_proj.weight, layer.down_proj.weight)
-    gates, ids = layer.route(xd.view(-1, H))
+    gates, ids = layer.route(xd.view(-1, H))               # training: the same batch again, so the same statistics and ids
     torch.cuda.synchronize()
     bx, by = oracle.BNState.fresh(r), oracle.BNState.fresh(r)
-    want_y, want_g, want_i = oracle.moe_forward(x, w, bx, by, k, training=False)
+    want_y, want_g, want_i = oracle.moe_forward(x, w, bx, by, k, training=training)
+    if training:
+        assert layer.router_norm_x.num_batches_tracked.item() == 2
     # the oracle's expert term for the ids the device chose (near-tied scores may resolve differently in bf16)
     want_e = oracle.expert_forward(x.view(-1, H), w.up_embed, w.down_embed, gates.cpu(), ids.cpu()).float()
     e_scale, m_scale = want_e.abs().max().item(), mlp.float().abs().max().item()
@@ -340,6 +345,43 @@ def test_layer_two_streams_equals_one_stream(dtype, device):
     s.synchronize()
     layer.overlap_branches = False
     assert torch.equal(out, layer(x * 2))
+
+
+def test_layer_copies_and_saves_like_a_plain_module(device, tmp_path):
+    """After a two-stream forward (side stream and events in use) a layer is still a plain nn.Module:
+    copy.deepcopy, torch.save / torch.load and a state_dict round trip give layers with identical output."""
+    import copy
+    from omni_moe.modules.omni_moe import OmniMoE, OmniMoEConfig
+    torch.manual_seed(3)
+    cfg = OmniMoEConfig(256, 512, "silu", 1024, 8)
+    layer = OmniMoE(cfg).to(device=device, dtype=torch.bfloat16).eval()
+    layer.overlap_min_work = 0
+    x = torch.randn(2, 200, 256, device=device).bfloat16()
+    want = layer(x)
+    twin = copy.deepcopy(layer)
+    assert torch.equal(twin(x), want)
+    path = str(tmp_path / "layer.pt")
+    torch.save(layer, path)
+    loaded = torch.load(path, weights_only=False)           # a file this test wrote itself
+    assert torch.equal(loaded(x), want)
+    fresh = OmniMoE(cfg).to(device=device, dtype=torch.bfloat16).eval()
+    fresh.load_state_dict(layer.state_dict())
+    fresh.overlap_min_work = 0
+    assert torch.equal(fresh(x), want)
+    assert not any(isinstance(v, (torch.cuda.Stream, torch.cuda.Event)) for v in vars(layer).values())
+
+
+def test_layer_takes_noncontiguous_weights(device):
+    """The reference's operators make every tensor argument contiguous (utils.py:47-65); the fused layer call does too."""
+    from omni_moe.modules.omni_moe import OmniMoE, OmniMoEConfig
+    torch.manual_seed(4)
+    layer = OmniMoE(OmniMoEConfig(128, 256, "silu", 256, 8)).to(device=device, dtype=torch.bfloat16).eval()
+    x = torch.randn(1, 300, 128, device=device).bfloat16()
+    want = layer(x)
+    w = layer.down_proj.weight.data
+    layer.down_proj.weight.data = w.t().contiguous().t()    # same values, column-major storage
+    assert not layer.down_proj.weight.is_contiguous()
+    assert torch.equal(layer(x), want)
 
 
 def test_add_inplace(device):

@@ -126,6 +126,8 @@ EXPERT_CASES = [
     # (T, H, N, k, dtype, kind)
     (1024, 1024, 1024, 32, torch.bfloat16, "ref"),      # reference benchmark grid (tests/test_expert.py:181-187)
     (1024, 1024, 4096, 32, torch.bfloat16, "ref"),
+    (1024, 1024, 16384, 32, torch.bfloat16, "ref"),     #   ... its two larger tables: 64 MiB and 256 MiB, where AUTO
+    (1024, 1024, 65536, 32, torch.bfloat16, "ref"),     #   goes back from the hidden-split to the gather algorithm
     (2048, 1024, 4096, 16, torch.bfloat16, "baseline"), # benchmark config 3 shape (token subset)
     (512, 256, 1024, 8, torch.float32, "baseline"),     # benchmark config 1 shape
     (256, 2048, 8192, 32, torch.bfloat16, "baseline"),  # benchmark config 5 row length
@@ -247,8 +249,7 @@ DENSE_CASES = [(16384, 1024, 256, 16, torch.bfloat16, "baseline"),   # the shape
 def test_expert_dense_algorithm(case, device):
     """The dense organisation for the reference's group regime (T*k/N > 256, omni_scheduler.py:58): a gate matrix and two
     MFMA GEMMs over all experts.  Same tolerance against the oracle; agreement with the gather algorithm to the 16
-    significant bits its coefficients carry; run-to-run identical; AUTO picks it under the reference's rule where the
-    experts are few enough (N <= 16 k)."""
+    significant bits its coefficients carry; run-to-run identical; AUTO never picks it (it touches unselected rows)."""
     from omni_moe.ops.hip import _lib
     T, H, N, k, dtype, kind = case
     x, up, down, gates, ids = _expert_inputs(T, H, N, k, dtype, kind, seed=T + H)
@@ -265,10 +266,35 @@ def test_expert_dense_algorithm(case, device):
     lib = _lib.load()
     auto_ws = lib.omni_expert_workspace_bytes(T, H, N, k, _lib.DTYPE_CODE[dtype], _lib.ALGO_AUTO)
     dense_ws = lib.omni_expert_workspace_bytes(T, H, N, k, _lib.DTYPE_CODE[dtype], _lib.ALGO_DENSE)
-    picks = T * k > 256 * N and N <= 16 * k              # the reference's group rule, and few enough experts for the GEMMs to pay
-    assert dense_ws > 0 and (auto_ws == dense_ws) == picks
-    if picks:
-        assert torch.equal(_ops().hip_omni_expert_func(*d), got)
+    assert dense_ws > 0 and auto_ws != dense_ws          # by name only
+
+
+def test_expert_unselected_nonfinite_rows(device):
+    """A table row that no token selects may hold anything: the reference only ever touches selected rows
+    (omni_expert.py:8-168 walks the scheduled pairs), and so do the gather, split and segment algorithms and
+    whatever AUTO picks -- also in the group regime (T*k/N > 256), where AUTO used to switch to the dense
+    algorithm.  The dense algorithm, by name, multiplies every token by every row: an Inf in an unselected
+    down row reaches every token (0 * Inf), which is the documented difference that keeps it out of AUTO."""
+    hip = _ops()
+    T, H, N, k = 8192, 256, 64, 8                          # 1024 pairs per expert: the group regime
+    g = torch.Generator().manual_seed(31)
+    x = torch.randn(T, H, generator=g).bfloat16()
+    up, down = ((torch.randn(N, H, generator=g) * 0.1).bfloat16() for _ in range(2))
+    gates = torch.rand(T, k, generator=g).bfloat16()
+    ids = torch.randint(0, N - 2, (T, k), generator=g, dtype=torch.int32)       # rows N-2 and N-1 are never selected
+    want = oracle.expert_forward(x, up, down, gates, ids)
+    up[N - 2, 5], up[N - 2, 9] = float("inf"), float("nan")
+    down[N - 1, 7] = float("inf")
+    d = [t.to(device) for t in (x, up, down, gates, ids)]
+    print("expert op with non-finite unselected rows", flush=True)
+    for algo in ("auto", "gather", "split", "segment"):
+        got = hip.hip_omni_expert_func(*d, algo=algo).cpu().float()
+        assert torch.isfinite(got).all(), algo
+        torch.testing.assert_close(got, want.float(), rtol=2e-2, atol=2e-2)
+    dense = hip.hip_omni_expert_func(*d, algo="dense").cpu().float()
+    assert not torch.isfinite(dense[:, 7]).any()           # the unselected Inf row poisons column 7 of every token
+    cols = [c for c in range(H) if c != 7]
+    torch.testing.assert_close(dense[:, cols], want.float()[:, cols], rtol=2e-2, atol=2e-2)   # the up-table Inf/NaN is masked by the zero gate
 
 
 def test_expert_dense_refusals_and_bad_ids(device):
