@@ -19,10 +19,15 @@ the library enqueues there).
   roofline_expert_hbm    the expert op at benchmark config 5's shape (2 GiB tables): HBM-resident, so
                          algorithmic bytes are HBM bytes
   kernels        per-launch figures for every stage
+  layer_c5       the whole layer at benchmark config 5 (32768 tokens, hidden 2048, intermediate 8192, 262144
+                 experts, top-32, Zipf-skewed keys): step time, tokens/s and its three MFMA GEMMs
+  ref_grid       the shapes of the reference's own operator benchmarks (tests/test_router.py:103-110,
+                 tests/test_expert.py:181-187, tests/test_mlp.py:144-150), each beside the same operator
+                 composed from torch library ops on this GPU
   cpu_baseline   the oracle (the reference's PyTorch layer restated with torch CPU ops) on the
                  host cores, same workload
 
-Sections (default: all): layer, kernels, expert_c3, expert_c5, probe, train, cpu.
+Sections (default: all): layer, kernels, expert_c3, expert_c5, layer_c5, ref_grid, probe, train, cpu.
 """
 import argparse
 import json
@@ -44,7 +49,7 @@ TRAFFIC_SOURCE = "profiles/bench_layer_c4_hbm_counters.txt, profiles/expert_c5_h
 TRAFFIC_BYTES = {"expert_c3": 180.6e6, "expert_c4": 57.8e6, "expert_gather_c3": 897.2e6, "gateup_c4": 134.4e6, "down_c4": 117.6e6,
                  "down_plain_c4": 109.2e6, "schedule_c3": 12.36e6,
                  "expert_c5_routed": 1029.2e6, "expert_c5_uniform": 8846.8e6}
-SECTIONS = ("layer", "kernels", "expert_c3", "expert_c5", "probe", "train", "cpu")
+SECTIONS = ("layer", "kernels", "expert_c3", "expert_c5", "layer_c5", "ref_grid", "probe", "train", "cpu")
 
 
 def expert_alg_bytes(T, H, k, s=2):
@@ -342,40 +347,52 @@ def main():
                                      note="x, dy (32 MiB each) and the tables are cache-resident"))
         del x3, up3, down3, g3, i3, y3
 
-    if "expert_c5" in sections:
-        # expert op at benchmark config 5's shape: 2 GiB of tables, so every selected row comes from HBM
-        T5, H5, N5, k5 = 32768, 2048, 262144, 32
+    if "expert_c5" in sections or "layer_c5" in sections:
+        # benchmark config 5: 32768 tokens, hidden 2048, intermediate 8192, 262144 experts (512 x 512 keys), top-32; 2 GiB of
+        # expert tables, so every selected row that is not reused comes from HBM.  Key popularity ~ Zipf(1.1) through
+        # eval-mode BatchNorm buffers (running_mean = 1.1 ln(1+i), running_var = 1 - eps: a per-key bias on the normalised
+        # logits; the reference's router has no bias of its own, omni_moe.py:47-52).  Weights are drawn on the device.
+        T5, H5, I5, N5, k5, r5 = 32768, 2048, 8192, 262144, 32, 512
         g = torch.Generator(device=dev).manual_seed(4)
-        x5 = torch.empty(T5, H5, device=dev, dtype=torch.bfloat16).normal_(0, 1, generator=g)
-        up5 = torch.empty(N5, H5, device=dev, dtype=torch.bfloat16).normal_(0, 0.02, generator=g)
-        down5 = torch.empty(N5, H5, device=dev, dtype=torch.bfloat16).normal_(0, 0.02, generator=g)
-        # ids and gates as the config-5 layer routes them: key popularity ~ Zipf(1.1) through eval-mode BatchNorm buffers
-        # (running_mean = 1.1 ln(1+i), running_var = 1 - eps: a per-key bias on the normalised logits)
-        r5 = 512
-        wx5 = torch.empty(r5, H5, device=dev, dtype=torch.bfloat16).normal_(0, 0.02, generator=g)
-        wy5 = torch.empty(r5, H5, device=dev, dtype=torch.bfloat16).normal_(0, 0.02, generator=g)
+        draw = lambda *shape, std: torch.empty(*shape, device=dev, dtype=torch.bfloat16).normal_(0, std, generator=g)
+        x5 = draw(T5, H5, std=1.0)
+        up5, down5 = draw(N5, H5, std=0.02), draw(N5, H5, std=0.02)
+        wx5, wy5 = draw(r5, H5, std=0.02), draw(r5, H5, std=0.02)
         rm = (1.1 * torch.log1p(torch.arange(r5, dtype=torch.float32))).to(device=dev, dtype=torch.bfloat16)
         rv = torch.full((r5,), 1.0 - 1e-5, device=dev, dtype=torch.bfloat16)
         g5, i5 = hip.hip_omni_router_fwd_func(x5, wx5, wy5, rm, rv, None, rm.clone(), rv.clone(), None, k5, training=False)
-        y5 = hip.hip_omni_expert_func(x5, up5, down5, g5, i5)
-        # oracle on 64 tokens, over the table rows they select
-        sub = 64
+        sub = 64                                          # tokens checked against the oracle, over the table rows they select
+
+        def expert_want5(gates, ids):
+            rows, inv = torch.unique(ids[:sub].long(), return_inverse=True)
+            return oracle.expert_forward(x5[:sub].cpu(), up5[rows].cpu(), down5[rows].cpu(), gates[:sub].cpu(), inv.cpu().to(torch.int32))
 
         def check5(y, gates, ids):
-            rows, inv = torch.unique(ids[:sub].long(), return_inverse=True)
-            want = oracle.expert_forward(x5[:sub].cpu(), up5[rows].cpu(), down5[rows].cpu(), gates[:sub].cpu(), inv.cpu().to(torch.int32))
-            torch.testing.assert_close(y[:sub].float().cpu(), want.float(), rtol=2e-2, atol=2e-2)
+            torch.testing.assert_close(y[:sub].float().cpu(), expert_want5(gates, ids).float(), rtol=2e-2, atol=2e-2)
 
+    if "expert_c5" in sections:
+        y5 = hip.hip_omni_expert_func(x5, up5, down5, g5, i5)
         check5(y5, g5, i5)
         used = torch.unique(i5).numel()
         counts = torch.bincount(i5.flatten().long(), minlength=N5)
         alg5 = expert_alg_bytes(T5, H5, k5)
-        m, b = time_launches(torch, lambda: hip.hip_omni_expert_func(x5, up5, down5, g5, i5), n=10, reps=5, warmup=2)
+        min5 = 2 * T5 * H5 * 2 + 2 * used * H5 * 2 + T5 * k5 * 6
+        skew = (f"the skewed router selects only {used} distinct experts (the most popular takes {int(counts.max())} of the {T5 * k5} pairs): "
+                "their rows stay in the caches, so few of the algorithmic bytes cross the fabric")
+        m, b = time_launches(torch, lambda: hip.hip_omni_expert_func(x5, up5, down5, g5, i5, algo="gather"), n=10, reps=5, warmup=2)
         kernels.append(hbm_entry("expert op (gather algorithm: expert_gather_kernel), config-5 shape (32768 tokens, hidden 2048, 262144 experts, top-32), "
-                                 "ids from the config-5 router (key popularity ~ Zipf(1.1))", m, b, alg5, TRAFFIC_BYTES["expert_c5_routed"],
-                                 2 * T5 * H5 * 2 + 2 * used * H5 * 2 + T5 * k5 * 6,
-                                 note=f"the skewed router selects only {used} distinct experts (the most popular takes {int(counts.max())} of the {T5 * k5} pairs): "
-                                      "their rows stay in the caches, so few of the algorithmic bytes cross the fabric"))
+                                 "ids from the config-5 router (key popularity ~ Zipf(1.1))", m, b, alg5, TRAFFIC_BYTES["expert_c5_routed"], min5, note=skew))
+        # the hidden-split algorithm on the same ids: which one wins depends on how many distinct rows are live, which the
+        # table size alone (all AUTO can see without a host sync) does not tell
+        ys = hip.hip_omni_expert_func(x5, up5, down5, g5, i5, algo="split")
+        check5(ys, g5, i5)
+        m_s, b_s = time_launches(torch, lambda: hip.hip_omni_expert_func(x5, up5, down5, g5, i5, algo="split"), n=10, reps=5, warmup=2)
+        kernels.append(hbm_entry("expert op (split algorithm: expert_split_dots_kernel + expert_split_accumulate_kernel), config-5 shape, "
+                                 "ids from the config-5 router (key popularity ~ Zipf(1.1))", m_s, b_s, alg5, TRAFFIC_BYTES.get("expert_c5_routed_split"), min5,
+                                 note="same inputs as the entry above, algo='split' by name (OmniMoE.expert_algo = 'split'): the live rows' column slices fit the XCDs' L2s"))
+        m_a, b_a = time_launches(torch, lambda: hip.hip_omni_expert_func(x5, up5, down5, g5, i5), n=10, reps=5, warmup=2)
+        out["expert_c5_routed"] = {"gather_ms": m, "split_ms": m_s, "auto_ms": m_a, "distinct_experts": used, "max_pairs_per_expert": int(counts.max()),
+                                   "note": "AUTO decides by table size (2 GiB: gather); the layer takes a hint (OmniMoE.expert_algo) where the id distribution is known"}
         # the same shape with ids spread evenly (32 distinct experts per token, uniform over all 262144): every selected
         # row comes from HBM, so algorithmic bytes are HBM bytes -- the case that shows the kernel against the HBM roofline
         iu = torch.randint(0, N5 // k5, (T5, k5), device=dev, generator=g, dtype=torch.int32) * k5 + torch.arange(k5, device=dev, dtype=torch.int32)
@@ -387,7 +404,122 @@ def main():
                        note="2 GiB of tables, no reuse to speak of: the rocprofv3 byte counters of this launch read the algorithmic bytes (profiles/expert_c5_hbm_counters.txt)")
         kernels.append(e5)
         out["roofline_expert_hbm"] = e5
-        del x5, up5, down5, g5, i5, y5, iu, yu
+        del y5, ys, iu, yu
+
+    if "layer_c5" in sections:
+        layer5 = OmniMoE(OmniMoEConfig(H5, I5, "silu", N5, k5))
+        layer5 = layer5.to(device=dev, dtype=torch.bfloat16).eval()
+        with torch.no_grad():
+            layer5.gate_proj.weight.copy_(draw(I5, H5, std=0.02)); layer5.up_proj.weight.copy_(draw(I5, H5, std=0.02))
+            layer5.down_proj.weight.copy_(draw(H5, I5, std=0.02))
+            layer5.router_gate_x.weight.copy_(wx5); layer5.router_gate_y.weight.copy_(wy5)
+            for bn in (layer5.router_norm_x, layer5.router_norm_y):
+                bn.running_mean.copy_(rm); bn.running_var.copy_(rv)
+        # the 2 GiB tables are the ones drawn above: the module's parameters alias them (no second copy in HBM)
+        layer5.up_embed.weight.data, layer5.down_embed.weight.data = up5, down5
+        per_algo = {}
+        for algo in ("auto", "split"):
+            layer5.expert_algo = algo
+            y5l = layer5(x5.view(8, T5 // 8, H5)).view(T5, H5)
+            # oracle on a token subset (eval mode is token-independent): router ids, then experts over the selected rows + MLP
+            bx = oracle.BNState(rm.float().cpu(), rv.float().cpu(), torch.zeros((), dtype=torch.long))
+            by = oracle.BNState(rm.float().cpu(), rv.float().cpu(), torch.zeros((), dtype=torch.long))
+            wg_, wi_, _ = oracle.router_forward(x5[:sub].cpu(), wx5.cpu(), wy5.cpu(), bx, by, k5, False)
+            agree = (i5[:sub].cpu().sort(-1).values == wi_.sort(-1).values).float().mean().item()
+            assert agree >= 0.99, agree
+            want5 = (oracle.mlp_forward(x5[:sub].cpu(), layer5.gate_proj.weight.cpu(), layer5.up_proj.weight.cpu(), layer5.down_proj.weight.cpu()).float()
+                     + expert_want5(g5, i5).float())
+            torch.testing.assert_close(y5l[:sub].float().cpu(), want5, rtol=2e-2, atol=2e-2)
+            m, b = time_launches(torch, lambda: layer5(x5.view(8, T5 // 8, H5)), n=5, reps=5, warmup=2)
+            per_algo[algo] = {"ms_per_step": m, "ms_per_step_best": b, "tokens_per_s": T5 / (m * 1e-3)}
+        layer5.expert_algo = "auto"
+        xf5 = x5
+        m_gu, b_gu = time_launches(torch, lambda: hip.hip_swiglu_linear_func(xf5, layer5.gate_proj.weight, layer5.up_proj.weight), n=5, reps=5, warmup=2)
+        e_gu = mfma_entry("gemm_nt_dma_kernel<swiglu> (gate/up projection + SwiGLU), config 5 (32768 x 2 x 8192 x 2048)", 4 * T5 * H5 * I5, m_gu, b_gu, None, sustained)
+        h5 = hip.hip_swiglu_linear_func(xf5, layer5.gate_proj.weight, layer5.up_proj.weight)
+        m_d, b_d = time_launches(torch, lambda: hip.hip_linear_func(h5, layer5.down_proj.weight), n=5, reps=5, warmup=2)
+        e_d = mfma_entry("gemm_nt_dma_kernel<plain> (down projection), config 5 (32768 x 2048 x 8192)", 2 * T5 * H5 * I5, m_d, b_d, None, sustained)
+        wcat5 = torch.cat([wx5, wy5], 0)
+        m_r, b_r = time_launches(torch, lambda: hip.hip_linear_func(xf5, wcat5), n=5, reps=5, warmup=2)
+        e_r = mfma_entry("gemm_nt_dma_kernel<plain> (router projection, both halves: 32768 x 1024 x 2048; arithmetic intensity 669 flop/B), config 5",
+                         4 * T5 * H5 * r5, m_r, b_r, None, sustained)
+        m_lib, _ = time_launches(torch, lambda: torch.matmul(xf5, wcat5.t()), n=5, reps=3, warmup=2)
+        e_r["library_gemm_same_flops_ms"] = m_lib
+        wcat_gu = torch.cat([layer5.gate_proj.weight, layer5.up_proj.weight], 0)
+        m_lib, _ = time_launches(torch, lambda: torch.matmul(xf5, wcat_gu.t()), n=5, reps=3, warmup=2)
+        e_gu["library_gemm_same_flops_ms"] = m_lib
+        del wcat_gu
+        m_lib, _ = time_launches(torch, lambda: torch.matmul(h5, layer5.down_proj.weight.t()), n=5, reps=3, warmup=2)
+        e_d["library_gemm_same_flops_ms"] = m_lib
+        m_rt, b_rt = time_launches(torch, lambda: layer5.route(xf5), n=5, reps=5, warmup=2)
+        kernels += [e_gu, e_d, e_r]
+        out["layer_c5"] = {"workload": "BASELINE.json configs[4] (benchmark config 5): full OmniMoE layer forward, 8x4096 tokens, hidden 2048, intermediate 8192, "
+                                       "262144 experts (512x512), top-32, eval-mode BatchNorm whose buffers carry the Zipf(1.1) key bias, seed 4",
+                           "ms_per_step": per_algo["auto"]["ms_per_step"], "tokens_per_s": per_algo["auto"]["tokens_per_s"],
+                           "with_expert_algo_split": per_algo["split"], "router_stage_ms": m_rt,
+                           "gate_up_TFLOPs": e_gu["achieved"], "down_TFLOPs": e_d["achieved"], "router_projection_TFLOPs": e_r["achieved"],
+                           "frac_of_mfma_peak": {"gate_up": e_gu["frac"], "down": e_d["frac"], "router_projection": e_r["frac"]},
+                           "checked": f"{sub} tokens against the oracle (router ids, experts over the selected rows, MLP) before timing"}
+        del layer5, h5, wcat5, y5l
+
+    if "expert_c5" in sections or "layer_c5" in sections:
+        del x5, up5, down5, wx5, wy5, g5, i5
+
+    if "ref_grid" in sections:
+        # The reference's own operator benchmarks (bf16, 1024 tokens), its flop conventions, each beside the same operator
+        # composed from torch library ops on this GPU (what the reference's harness calls the PyTorch implementation).
+        grid = []
+        Tg = 1024
+        gen = torch.Generator(device=dev).manual_seed(0)
+        for r_, k_ in ((64, 16), (64, 32), (128, 16), (128, 32), (256, 16), (256, 32)):        # tests/test_router.py:103-110
+            lx = torch.log_softmax(torch.randn(Tg, r_, device=dev, generator=gen), -1).bfloat16()
+            ly = torch.log_softmax(torch.randn(Tg, r_, device=dev, generator=gen), -1).bfloat16()
+            sc, ix = hip.hip_omni_router_func(lx, ly, r_, k_)
+            ws_, wi_ = oracle.router_select(lx[:64].cpu(), ly[:64].cpu(), r_, k_)
+            assert torch.equal(ix[:64].cpu(), wi_) and torch.equal(sc[:64].cpu().float(), ws_.float())
+            m, b = time_launches(torch, lambda: hip.hip_omni_router_func(lx, ly, r_, k_))
+            mt, _ = time_launches(torch, lambda: (lx[:, :, None] + ly[:, None, :]).view(Tg, -1).topk(k_, dim=-1), n=10, reps=3, warmup=2)
+            grid.append({"op": "router", "tokens": Tg, "num_keys": r_, "top_k": k_, "ms": m, "ms_best": b, "torch_ops_ms": mt, "speedup": mt / m,
+                         "TFLOPs_reference_convention": 4.0 * Tg * r_ * r_ / (m * 1e-3) / 1e12})
+        for N_ in (1024, 4096, 16384, 65536):                                                  # tests/test_expert.py:181-187
+            k_ = 32
+            xg = torch.empty(Tg, 1024, device=dev, dtype=torch.bfloat16).normal_(0, 0.5, generator=gen)
+            ug = torch.empty(N_, 1024, device=dev, dtype=torch.bfloat16).normal_(0, 0.1, generator=gen)
+            vg = torch.empty(N_, 1024, device=dev, dtype=torch.bfloat16).normal_(0, 0.1, generator=gen)
+            gg = torch.empty(Tg, k_, device=dev, dtype=torch.bfloat16).normal_(0, 0.1, generator=gen)
+            ig = torch.randint(0, N_, (Tg, k_), device=dev, dtype=torch.int32, generator=gen)
+            yg = hip.hip_omni_expert_func(xg, ug, vg, gg, ig)
+            rows, inv = torch.unique(ig[:64].long(), return_inverse=True)
+            wantg = oracle.expert_forward(xg[:64].cpu(), ug[rows].cpu(), vg[rows].cpu(), gg[:64].cpu(), inv.cpu().to(torch.int32))
+            torch.testing.assert_close(yg[:64].float().cpu(), wantg.float(), rtol=2e-2, atol=2e-2)
+            m, b = time_launches(torch, lambda: hip.hip_omni_expert_func(xg, ug, vg, gg, ig))
+
+            def torch_expert():
+                il = ig.long()
+                sc_ = torch.einsum("th,tkh->tk", xg, ug[il])
+                return torch.einsum("tk,tkh->th", torch.nn.functional.silu(sc_) * gg, vg[il])
+
+            mt, _ = time_launches(torch, torch_expert, n=10, reps=3, warmup=2)
+            grid.append({"op": "expert", "tokens": Tg, "hidden": 1024, "num_experts": N_, "top_k": k_, "ms": m, "ms_best": b, "torch_ops_ms": mt, "speedup": mt / m,
+                         "TFLOPs_reference_convention": 4.0 * Tg * k_ * 1024 / (m * 1e-3) / 1e12,
+                         "algorithmic_GBs": expert_alg_bytes(Tg, 1024, k_) / (m * 1e-3) / 1e9})
+            del xg, ug, vg, gg, ig, yg
+        gen = torch.Generator(device=dev).manual_seed(42)
+        for I_ in (1024, 4096, 16384, 65536):                                                  # tests/test_mlp.py:144-150
+            xg = torch.empty(Tg, 1024, device=dev, dtype=torch.bfloat16).normal_(0, 0.5, generator=gen)
+            wg_ = torch.empty(I_, 1024, device=dev, dtype=torch.bfloat16).normal_(0, 0.1, generator=gen)
+            wu_ = torch.empty(I_, 1024, device=dev, dtype=torch.bfloat16).normal_(0, 0.1, generator=gen)
+            wd_ = torch.empty(1024, I_, device=dev, dtype=torch.bfloat16).normal_(0, 0.1, generator=gen)
+            yg = hip.hip_omni_mlp_func(xg, wg_, wu_, wd_)
+            wantg = oracle.mlp_forward(xg[:32].cpu().float(), wg_.cpu().float(), wu_.cpu().float(), wd_.cpu().float())
+            scale = max(wantg.abs().max().item(), 1.0)
+            torch.testing.assert_close(yg[:32].float().cpu() / scale, wantg / scale, rtol=2e-2, atol=2e-2)
+            m, b = time_launches(torch, lambda: hip.hip_omni_mlp_func(xg, wg_, wu_, wd_), n=20)
+            mt, _ = time_launches(torch, lambda: torch.matmul(torch.nn.functional.silu(torch.matmul(xg, wg_.t())) * torch.matmul(xg, wu_.t()), wd_.t()), n=10, reps=3, warmup=2)
+            grid.append({"op": "mlp", "tokens": Tg, "hidden": 1024, "intermediate": I_, "ms": m, "ms_best": b, "torch_ops_ms": mt, "speedup": mt / m,
+                         "TFLOPs_reference_convention": 6.0 * Tg * 1024 * I_ / (m * 1e-3) / 1e12})
+            del xg, wg_, wu_, wd_, yg
+        out["ref_grid"] = grid
 
     if kernels:
         out["kernels"] = kernels

@@ -307,6 +307,26 @@ OMNI_API int32_t omni_moe_fwd(const void* x, const void* gate_weight, const void
                               int32_t training, float momentum, float eps, void* workspace, void* stream,
                               void* side_stream, void* fork_event, void* join_event);
 
+/* omni_moe_fwd with the expert algorithm named by the caller (OMNI_EXPERT_ALGO_*; omni_moe_fwd is this call with
+ * OMNI_EXPERT_ALGO_AUTO).  AUTO decides from sizes alone, without a device-to-host read; which algorithm is faster
+ * also depends on how many DISTINCT experts the router picks, which only the caller can know: with tables far beyond
+ * the caches but a skewed router (benchmark config 5: 2 GiB of tables, ~3700 live experts) SPLIT serves the live
+ * rows from the XCDs' L2s where AUTO's GATHER fetches them over the fabric.  An algorithm that does not cover the
+ * shape is OMNI_ERR_UNSUPPORTED before anything is enqueued.  The workspace size depends on the algorithm.
+ * No counterpart in the reference (its scheduler reads the id statistics back to the host, omni_scheduler.py:82,90). */
+OMNI_API size_t omni_moe_workspace_bytes_algo(int64_t num_tokens, int32_t hidden_size, int32_t intermediate_size,
+                                              int64_t num_experts, int32_t num_expert_sqrt, int32_t num_experts_per_token,
+                                              int32_t dtype, int32_t expert_algo);
+OMNI_API int32_t omni_moe_fwd_algo(const void* x, const void* gate_weight, const void* up_weight, const void* down_weight,
+                                   const void* router_weight_x, const void* router_weight_y,
+                                   void* running_mean_x, void* running_var_x, int64_t* num_batches_tracked_x,
+                                   void* running_mean_y, void* running_var_y, int64_t* num_batches_tracked_y,
+                                   const void* up_embed, const void* down_embed, void* y,
+                                   int64_t num_tokens, int32_t hidden_size, int32_t intermediate_size, int64_t num_experts,
+                                   int32_t num_expert_sqrt, int32_t num_experts_per_token, int32_t dtype, int32_t stats_dtype,
+                                   int32_t training, float momentum, float eps, void* workspace, void* stream,
+                                   void* side_stream, void* fork_event, void* join_event, int32_t expert_algo);
+
 #ifdef __cplusplus
 }
 #endif

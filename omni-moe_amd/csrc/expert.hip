@@ -539,6 +539,17 @@ static int resolve_algo(int algo, int64_t T, int H, int64_t N, int k, int dtype)
   return OMNI_EXPERT_ALGO_GATHER;
 }
 
+// OMNI_OK when omni_expert_fwd takes `algo` for these sizes (what the whole-layer call checks before it enqueues anything).
+int expert_algo_check(int algo, int64_t T, int H, int64_t N, int k, int dtype) {
+  const int es = dtype == OMNI_F32 ? 4 : 2;
+  switch (algo) {
+    case OMNI_EXPERT_ALGO_AUTO: case OMNI_EXPERT_ALGO_GATHER: case OMNI_EXPERT_ALGO_SEGMENT: return OMNI_OK;
+    case OMNI_EXPERT_ALGO_SPLIT: return (split_lanes_per_row(H, es) != 0 && k <= 2 * kWave) ? OMNI_OK : OMNI_ERR_UNSUPPORTED;
+    case OMNI_EXPERT_ALGO_DENSE: return (k == 0 || T == 0 || dense_covers(T, H, N, k, dtype)) ? OMNI_OK : OMNI_ERR_UNSUPPORTED;
+    default: return OMNI_ERR_UNSUPPORTED;
+  }
+}
+
 }  // namespace omni
 
 extern "C" OMNI_API size_t omni_expert_workspace_bytes(int64_t num_tokens, int32_t hidden_size, int64_t num_experts,

@@ -9,18 +9,27 @@
 namespace omni {
 static inline size_t up256(size_t v) { return (v + 255) / 256 * 256; }
 static inline size_t elem_bytes(int dtype) { return dtype == OMNI_F32 ? 4 : 2; }
+// defined beside the expert kernels: OMNI_OK when omni_expert_fwd takes `algo` at this shape (decided from the sizes alone)
+int expert_algo_check(int algo, int64_t num_tokens, int hidden_size, int64_t num_experts, int top_k, int dtype);
 }  // namespace omni
 
 // workspace: router workspace | gates [T,k] | ids [T,k] | expert output [T,H] | expert workspace | SwiGLU activations [T,I]
 extern "C" OMNI_API size_t omni_moe_workspace_bytes(int64_t num_tokens, int32_t hidden_size, int32_t intermediate_size,
                                                     int64_t num_experts, int32_t num_expert_sqrt, int32_t num_experts_per_token,
                                                     int32_t dtype) {
+  return omni_moe_workspace_bytes_algo(num_tokens, hidden_size, intermediate_size, num_experts, num_expert_sqrt, num_experts_per_token,
+                                       dtype, OMNI_EXPERT_ALGO_AUTO);
+}
+
+extern "C" OMNI_API size_t omni_moe_workspace_bytes_algo(int64_t num_tokens, int32_t hidden_size, int32_t intermediate_size,
+                                                         int64_t num_experts, int32_t num_expert_sqrt, int32_t num_experts_per_token,
+                                                         int32_t dtype, int32_t expert_algo) {
   using namespace omni;
   if (num_tokens < 0 || hidden_size <= 0 || intermediate_size <= 0 || num_expert_sqrt <= 0 || num_experts_per_token < 0) return 0;
   const size_t es = elem_bytes(dtype), T = (size_t)num_tokens, k = (size_t)num_experts_per_token;
   return up256(omni_router_workspace_bytes(num_tokens, num_expert_sqrt, dtype)) + up256(T * k * es) + up256(T * k * 4) +
          up256(T * (size_t)hidden_size * es) +
-         up256(omni_expert_workspace_bytes(num_tokens, hidden_size, num_experts, num_experts_per_token, dtype, OMNI_EXPERT_ALGO_AUTO)) +
+         up256(omni_expert_workspace_bytes(num_tokens, hidden_size, num_experts, num_experts_per_token, dtype, expert_algo)) +
          up256(omni_mlp_workspace_bytes(num_tokens, hidden_size, intermediate_size, dtype));
 }
 
@@ -33,6 +42,22 @@ extern "C" OMNI_API int32_t omni_moe_fwd(const void* x, const void* gate_weight,
                                          int32_t num_expert_sqrt, int32_t num_experts_per_token, int32_t dtype, int32_t stats_dtype,
                                          int32_t training, float momentum, float eps, void* workspace, void* stream,
                                          void* side_stream, void* fork_event, void* join_event) {
+  return omni_moe_fwd_algo(x, gate_weight, up_weight, down_weight, router_weight_x, router_weight_y, running_mean_x, running_var_x,
+                           num_batches_tracked_x, running_mean_y, running_var_y, num_batches_tracked_y, up_embed, down_embed, y,
+                           num_tokens, hidden_size, intermediate_size, num_experts, num_expert_sqrt, num_experts_per_token, dtype,
+                           stats_dtype, training, momentum, eps, workspace, stream, side_stream, fork_event, join_event,
+                           OMNI_EXPERT_ALGO_AUTO);
+}
+
+extern "C" OMNI_API int32_t omni_moe_fwd_algo(const void* x, const void* gate_weight, const void* up_weight, const void* down_weight,
+                                              const void* router_weight_x, const void* router_weight_y,
+                                              void* running_mean_x, void* running_var_x, int64_t* num_batches_tracked_x,
+                                              void* running_mean_y, void* running_var_y, int64_t* num_batches_tracked_y,
+                                              const void* up_embed, const void* down_embed, void* y,
+                                              int64_t num_tokens, int32_t hidden_size, int32_t intermediate_size, int64_t num_experts,
+                                              int32_t num_expert_sqrt, int32_t num_experts_per_token, int32_t dtype, int32_t stats_dtype,
+                                              int32_t training, float momentum, float eps, void* workspace, void* stream,
+                                              void* side_stream, void* fork_event, void* join_event, int32_t expert_algo) {
   using namespace omni;
   if (num_tokens < 0 || hidden_size <= 0 || intermediate_size <= 0 || num_experts <= 0 || num_expert_sqrt <= 0) return OMNI_ERR_SHAPE;
   if (dtype != OMNI_BF16 && dtype != OMNI_F16 && dtype != OMNI_F32) return OMNI_ERR_DTYPE;
@@ -43,6 +68,7 @@ extern "C" OMNI_API int32_t omni_moe_fwd(const void* x, const void* gate_weight,
     if (k < 0 || k > r * r || k > 128 || k % 2 != 0) return OMNI_ERR_TOPK;
     if (r > 1024 || hidden_size * esz > 8192) return OMNI_ERR_UNSUPPORTED;
     if (r * r > num_experts) return OMNI_ERR_SHAPE;                                                   // ids reach r*r - 1
+    if (int e = expert_algo_check(expert_algo, num_tokens, hidden_size, num_experts, num_experts_per_token, dtype)) return e;
   }
   if (num_tokens == 0) return OMNI_OK;
   if (training && num_tokens == 1) return OMNI_ERR_SHAPE;   // batch statistics of one sample: nn.BatchNorm1d raises
@@ -56,7 +82,7 @@ extern "C" OMNI_API int32_t omni_moe_fwd(const void* x, const void* gate_weight,
   int32_t* ids = (int32_t*)w;  w += up256(T * k * 4);
   void* experts = w;    w += up256(T * (size_t)hidden_size * es);
   void* expert_ws = w;
-  w += up256(omni_expert_workspace_bytes(num_tokens, hidden_size, num_experts, num_experts_per_token, dtype, OMNI_EXPERT_ALGO_AUTO));
+  w += up256(omni_expert_workspace_bytes(num_tokens, hidden_size, num_experts, num_experts_per_token, dtype, expert_algo));
   void* h = w;
 
   hipStream_t main_s = (hipStream_t)stream;
@@ -73,7 +99,7 @@ extern "C" OMNI_API int32_t omni_moe_fwd(const void* x, const void* gate_weight,
                           num_tokens, hidden_size, num_expert_sqrt, num_experts_per_token, dtype, stats_dtype, router_ws, branch);
   if (!e) e = omni_swiglu_linear_fwd(x, gate_weight, up_weight, h, num_tokens, hidden_size, intermediate_size, dtype, main_s);
   if (!e) e = omni_expert_fwd(x, up_embed, down_embed, gates, ids, experts, num_tokens, hidden_size, num_experts,
-                              num_experts_per_token, dtype, OMNI_EXPERT_ALGO_AUTO, expert_ws, branch);
+                              num_experts_per_token, dtype, expert_algo, expert_ws, branch);
   if (!side_stream) {   // one stream: the add is the down projection's epilogue
     if (!e) e = omni_linear_fwd(h, down_weight, experts, y, num_tokens, intermediate_size, hidden_size, dtype, main_s);
     return e;

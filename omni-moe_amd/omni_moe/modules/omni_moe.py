@@ -98,6 +98,10 @@ class OmniMoE(nn.Module):
     # The fork and join cost about 50 us of host time per call, so below this much work (tokens x hidden x
     # intermediate; 2048 x 1024 x 4096 measured level on an MI355X) the call would be host-bound: one stream then.
     overlap_min_work = 2 ** 33
+    # Expert algorithm of the fused forward: "auto" decides from the sizes alone (no device-to-host read).  Which one is
+    # faster also depends on how many DISTINCT experts the router picks: with tables far beyond the caches and a skewed
+    # router (few live experts) "split" beats auto's "gather"; the caller who knows the distribution says so here.
+    expert_algo = "auto"
 
     @staticmethod
     def _branch_resources(device):
@@ -142,5 +146,5 @@ class OmniMoE(nn.Module):
                 ny.running_mean, ny.running_var, ny.num_batches_tracked,
                 self.up_embed.weight, self.down_embed.weight, self.top_k,
                 training=self.training, momentum=nx.momentum, eps=nx.eps,
-                side_stream=side, fork_event=fork, join_event=join)
+                side_stream=side, fork_event=fork, join_event=join, expert_algo=self.expert_algo)
         return out.view(bsz, seq_len, -1)

@@ -576,10 +576,12 @@ def hip_omni_moe_fwd_func(
     num_experts_per_token: int, training: bool, momentum: float = 0.1, eps: float = 1e-5,
     side_stream: Optional["torch.cuda.Stream"] = None,
     fork_event: Optional["torch.cuda.Event"] = None, join_event: Optional["torch.cuda.Event"] = None,
+    expert_algo: str = "auto",
 ) -> torch.Tensor:
     """The whole layer forward (reference omni_moe.py:60-106) for ``x`` of shape (tokens, hidden) in one
     library call.  With ``side_stream`` (and two events) the router + expert branch is enqueued next
-    to the MLP branch; the current stream waits for it before the final add."""
+    to the MLP branch; the current stream waits for it before the final add.  ``expert_algo`` names the
+    expert algorithm ("auto" decides from the sizes alone)."""
     T, H = x.shape
     I, N, r, k = gate_weight.size(0), up_embed.size(0), router_weight_x.size(0), int(num_experts_per_token)
     weights = (gate_weight, up_weight, down_weight, router_weight_x, router_weight_y, up_embed, down_embed)
@@ -603,18 +605,21 @@ def hip_omni_moe_fwd_func(
     lib = _lib.load()
     dt = _lib.DTYPE_CODE[x.dtype]
     y = torch.empty_like(x)
-    ws = torch.empty(max(lib.omni_moe_workspace_bytes(T, H, I, N, r, k, dt), 1), device=dev, dtype=torch.uint8)
+    if expert_algo not in _ALGOS:
+        raise ValueError(f"expert_algo must be one of {sorted(_ALGOS)}")
+    al = _ALGOS[expert_algo]
+    ws = torch.empty(max(lib.omni_moe_workspace_bytes_algo(T, H, I, N, r, k, dt, al), 1), device=dev, dtype=torch.uint8)
     side = fork = join = 0
     if side_stream is not None:
         side, fork, join = side_stream.cuda_stream, fork_event.cuda_event, join_event.cuda_event
     with torch.cuda.device(dev):
-        code = lib.omni_moe_fwd(
+        code = lib.omni_moe_fwd_algo(
             _lib.ptr(x), _lib.ptr(gate_weight), _lib.ptr(up_weight), _lib.ptr(down_weight), _lib.ptr(router_weight_x),
             _lib.ptr(router_weight_y), _lib.ptr(running_mean_x), _lib.ptr(running_var_x), _lib.ptr(num_batches_tracked_x),
             _lib.ptr(running_mean_y), _lib.ptr(running_var_y), _lib.ptr(num_batches_tracked_y), _lib.ptr(up_embed),
             _lib.ptr(down_embed), _lib.ptr(y), T, H, I, N, r, k, dt, _lib.DTYPE_CODE[running_mean_x.dtype],
-            1 if training else 0, float(momentum), float(eps), _lib.ptr(ws), _lib.stream_ptr(), side, fork, join)
-    _lib.check(code, "omni_moe_fwd")
+            1 if training else 0, float(momentum), float(eps), _lib.ptr(ws), _lib.stream_ptr(), side, fork, join, al)
+    _lib.check(code, "omni_moe_fwd_algo")
     # ws is released here: the current stream has been made to wait for the side branch, so every
     # later use of that memory (allocated from this stream's pool) is ordered after both branches
     return y

@@ -286,7 +286,8 @@ def test_layer_expert_term_visible_auto_split(two_streams, dtype, training, devi
     from omni_moe.modules.omni_moe import OmniMoE, OmniMoEConfig
     T, H, I, N, k = 4096, 512, 512, (1024 if dtype == torch.float32 else 4096), 8
     x, w = oracle.make_layer_inputs(21, T, H, I, N, dtype=dtype, w_std=0.1)
-    w.down_proj = (w.down_proj.float() * 0.03).to(dtype)     # the shared MLP scaled down to the size of the expert term
+    # the shared MLP scaled down to the size of the expert term (batch statistics flatten the gates: smaller still in training)
+    w.down_proj = (w.down_proj.float() * (0.006 if training else 0.03)).to(dtype)
     r = w.router_gate_x.size(0)
     layer = OmniMoE(OmniMoEConfig(H, I, "silu", N, k))
     layer.load_state_dict({"gate_proj.weight": w.gate_proj, "up_proj.weight": w.up_proj, "down_proj.weight": w.down_proj,
@@ -313,7 +314,7 @@ def test_layer_expert_term_visible_auto_split(two_streams, dtype, training, devi
     want_e = oracle.expert_forward(x.view(-1, H), w.up_embed, w.down_embed, gates.cpu(), ids.cpu()).float()
     e_scale, m_scale = want_e.abs().max().item(), mlp.float().abs().max().item()
     print(f"   max |experts| {e_scale:.3f}, max |mlp| {m_scale:.3f}")
-    assert e_scale > 0.2 * m_scale                             # the expert term is visible
+    assert e_scale > 0.15 * m_scale                            # the expert term is visible (batch statistics spread the gates a little thinner)
     got_e = (y.float() - mlp.float()).cpu()
     tol = 1e-4 if dtype == torch.float32 else 2e-2            # bf16: y and mlp are rounded to bf16 on the scale of their sum
     assert (got_e - want_e).abs().max().item() <= tol * (e_scale + m_scale), (got_e - want_e).abs().max().item()
