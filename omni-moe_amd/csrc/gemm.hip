@@ -73,6 +73,7 @@ struct GemmArgs {           // all element offsets below are scaled by the eleme
   const float* gate;      // kEpiGate only: [M, N] fp32 factors; C is then [M, 2N]: round(v) in columns 0..N-1, round(v - round(v)) in N..2N-1
   uint8_t* save_gate;     // kEpiSwiglu only, or NULL: [M, N] the rounded gate and up projections, kept for a backward pass
   uint8_t* save_up;       //   (16-byte stores only: N % 8 == 0)
+  int exclusive;          // nothing is meant to run beside this launch: the 256 x 256 tile may take the streaming form, which holds every CU
 };
 
 // Which output tile a block owns.  Blocks go round-robin over the 8 XCDs; each XCD gets
@@ -626,11 +627,177 @@ __global__ __launch_bounds__(NW * 64, 1) void gemm_nt_dma_kernel(const GemmArgs 
   gemm_epilogue<DT, TM, TN, EPI>(g, acc, m0, n0, wm, wn, lane);
 }
 
+// ---- the 256 x 256 tile as a stream over several output tiles ----------------------------------------
+// One block per CU walks its share of the output tiles (tile index blockIdx, blockIdx + gridDim, ...).  The K tiles of
+// consecutive output tiles form ONE stream through the two LDS stages: while a block multiplies the last K tiles of an
+// output tile, the first K tiles of its next one are already on their way, so only a block's first output tile waits for
+// memory before its first matrix instruction (gate/up projection at 4096 x 4096 x 1024, two tiles per block: 62.9 us
+// against 65.3 us; 32768 x 16384 x 2048: 1.82 against 1.87 ms).  Ring loads are buffer loads (scalar base and tile
+// offsets, one 32-bit lane offset per operand).  The grid keeps every CU until the kernel ends, so a kernel on another
+// stream finds no room beside it: the callers use this form where nothing is meant to run concurrently.
+// Needs full tiles (M % 256 == 0, N a multiple of the tile's columns), K % 64 == 0, whole rounds of 256 tiles.
+__device__ __forceinline__ void tile_coords_of(const GemmArgs& g, int b, int& tile_m, int& tile_n) {
+  if (g.patch_m > 0) {
+    const int per_patch = g.patch_m * g.patch_n;
+    const int xcd = b & 7, idx = b >> 3;
+    const int patch = (idx / per_patch) * 8 + xcd, within = idx % per_patch;
+    const int patches_m = g.tiles_m / g.patch_m;
+    tile_m = (patch % patches_m) * g.patch_m + within % g.patch_m;
+    tile_n = (patch / patches_m) * g.patch_n + within / g.patch_m;
+  } else {
+    tile_m = b % g.tiles_m;
+    tile_n = b / g.tiles_m;
+  }
+}
+
+template <int DT, int EPI>
+__global__ __launch_bounds__(512, 1) void gemm_stream_kernel(const GemmArgs g) {
+  constexpr int TM = 4, TN = 2;                      // 8 waves as 2 x 4, each 128 x 64
+  constexpr int BM = 256, BR = 256;
+  constexpr int BN = (EPI == kEpiSwiglu) ? 128 : 256;
+  constexpr int kRow = 128, kStage = (BM + BR) * kRow;
+  extern __shared__ __align__(16) uint8_t lds[];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave & 1, wn = wave >> 1;
+  const int num_kt = g.K / 64;
+  const int num_tiles = g.tiles_m * g.tiles_n;
+  const uint32_t row_bytes = (uint32_t)g.K * 2;
+
+  const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc((void*)g.a, 0, 0x7fffffff, 0x00020000);
+  const uint8_t* bsel = (EPI == kEpiSwiglu && (wave >> 2)) ? g.b1 : g.b0;      // waves 0-3 fetch gate rows, 4-7 the up rows
+  const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc((void*)bsel, 0, 0x7fffffff, 0x00020000);
+
+  // Load instruction p of a wave fills LDS rows (8p + wave)*8 + lane/8 of a tile; the lane fetches the logical chunk that
+  // belongs at its (swizzled) position, which depends on the wave's parity and the lane only.  For the SwiGLU form rows
+  // 64p .. 64p+31 of the weight tile are gate rows and 64p+32 .. 64p+63 the matching up rows of wave column p.
+  const int sw = (lane & 7) ^ ((4 * (wave & 1) + (lane >> 4)) & 7);
+  const uint32_t a_voff = (uint32_t)(wave * 8 + (lane >> 3)) * row_bytes + sw * 16;
+  const uint32_t b_voff = (uint32_t)((EPI == kEpiSwiglu ? (wave & 3) * 8 : wave * 8) + (lane >> 3)) * row_bytes + sw * 16;
+  constexpr int kBRowsPerInstr = (EPI == kEpiSwiglu) ? 32 : 64;     // weight rows between consecutive load instructions of a wave
+
+  // fetch cursor: the next K tile of the stream to request
+  int f_tile = blockIdx.x, f_kt = 0, f_stage = 0;
+  bool half_pending = false;                          // the cursor's K tile has its activation half requested, not yet its weights
+  uint32_t f_a = 0, f_b = 0;                          // byte offsets of the tile's first activation / weight row
+  auto cursor_coords = [&]() {
+    int tm, tn;
+    tile_coords_of(g, f_tile, tm, tn);
+    f_a = (uint32_t)(tm * BM) * row_bytes;
+    f_b = (uint32_t)(tn * BN) * row_bytes;
+  };
+  cursor_coords();
+  auto issue_one = [&](int q) __attribute__((always_inline)) {       // q = 0..3: activation rows, 4..7: weight rows
+    uint8_t* st = lds + f_stage * kStage;
+    if (q < 4)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (__attribute__((address_space(3))) void*)(st + (8 * q + wave) * 1024), 16, a_voff,
+                                               f_a + (uint32_t)(q * 64) * row_bytes + f_kt * 128, 0, 0);
+    else
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (__attribute__((address_space(3))) void*)(st + BM * kRow + (8 * (q - 4) + wave) * 1024), 16, b_voff,
+                                               f_b + (uint32_t)((q - 4) * kBRowsPerInstr) * row_bytes + f_kt * 128, 0, 0);
+  };
+  auto cursor_advance = [&]() {                        // after a K tile's second half has been issued
+    f_stage ^= 1;
+    if (++f_kt == num_kt) {
+      f_kt = 0;
+      f_tile += gridDim.x;
+      if (f_tile < num_tiles) cursor_coords();
+    }
+  };
+
+  // fragment reads: lane reads row lane%32, logical chunk 2*slab + lane/32, into buffer slab&1
+  const int rl = lane & 31;
+  int off_slab[4];
+#pragma unroll
+  for (int sl = 0; sl < 4; ++sl) off_slab[sl] = rl * kRow + swizzle<64>(rl, 2 * sl + (lane >> 5)) * 16;
+  const int a_frag = (wm * TM * 32) * kRow, b_frag = BM * kRow + (wn * TN * 32) * kRow;
+  u32x4_t af[2][TM], bf[2][TN];
+  auto read_one = [&](int stage, int slab, int f) __attribute__((always_inline)) {
+    const uint8_t* st = lds + stage * kStage + off_slab[slab];
+    if (f < TM) af[slab & 1][f] = *(const u32x4_t*)(st + a_frag + f * 32 * kRow);
+    else bf[slab & 1][f - TM] = *(const u32x4_t*)(st + b_frag + (f - TM) * 32 * kRow);
+  };
+
+  f32x16_t acc[TM][TN];
+  auto clear_acc = [&]() __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int q = 0; q < 16; ++q) acc[i][j][q] = 0.f;
+  };
+  clear_acc();
+
+  // One slab: TM*TN matrix instructions, each followed by at most two memory instructions: the fragment reads of the
+  // following slab (stage read_stage) and, dma = 1 / 2, the activation / weight loads of the cursor's K tile.
+  auto slab = [&](auto sl_tag, auto next_tag, auto dma_tag, int read_stage) __attribute__((always_inline)) {
+    constexpr int sl = decltype(sl_tag)::value, next_slab = decltype(next_tag)::value, dma = decltype(dma_tag)::value;
+    const bool fv = dma == 1 ? f_tile < num_tiles : (dma == 2 && half_pending);
+#pragma unroll
+    for (int ij = 0; ij < TM * TN; ++ij) {
+      const int i = ij / TN, j = ij % TN;
+      acc[i][j] = mfma32<DT>(bf[sl & 1][j], af[sl & 1][i], acc[i][j]);
+      __builtin_amdgcn_sched_barrier(0);
+      if (ij < TM + TN) read_one(read_stage, next_slab, ij);
+      if constexpr (dma != 0) {
+        if (ij >= TM + TN) {
+          const int q0 = (dma == 1 ? 0 : 4) + (ij - (TM + TN)) * 2;
+          if (fv) { issue_one(q0); issue_one(q0 + 1); }
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  using I0 = std::integral_constant<int, 0>; using I1 = std::integral_constant<int, 1>;
+  using I2 = std::integral_constant<int, 2>; using I3 = std::integral_constant<int, 3>;
+  int c_stage = 0;                                     // stage of the K tile being multiplied
+  // one K tile; on entry its slab-0 fragments are in registers
+  auto k_tile = [&]() __attribute__((always_inline)) {
+    slab(I0{}, I1{}, I2{}, c_stage);                   // the weights of the K tile whose activations were requested one slab ago
+    if (half_pending) { cursor_advance(); half_pending = false; }
+    slab(I1{}, I2{}, I0{}, c_stage);
+    slab(I2{}, I3{}, I0{}, c_stage);
+    wait_lds_reads();                                  // this wave holds every fragment of the K tile
+    wait_vmcnt<0>();                                   // the next K tile has landed
+    __builtin_amdgcn_s_barrier();                      // ... for all waves; this K tile's stage is free
+    __builtin_amdgcn_sched_barrier(0);
+    half_pending = f_tile < num_tiles;
+    slab(I3{}, I0{}, I1{}, c_stage ^ 1);               // the activations of the K tile two ahead go into the freed stage
+    c_stage ^= 1;
+  };
+
+  // ---- prologue: the stream's first two K tiles
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+#pragma unroll
+    for (int q = 0; q < 8; ++q) issue_one(q);
+    cursor_advance();
+  }
+  wait_vmcnt<8>();                                     // the first K tile has landed
+  __builtin_amdgcn_s_barrier();
+#pragma unroll
+  for (int f = 0; f < TM + TN; ++f) read_one(0, 0, f);
+
+  for (int tile = blockIdx.x; tile < num_tiles; tile += gridDim.x) {
+    for (int kt = 0; kt < num_kt; ++kt) k_tile();
+    int tm, tn;
+    tile_coords_of(g, tile, tm, tn);
+    gemm_epilogue<DT, TM, TN, EPI>(g, acc, tm * BM, tn * BN, wm, wn, lane);
+    clear_acc();
+  }
+}
+
 // One list entry per kernel instantiation that launch_gemm can start (the static members come into being
 // at library load for every instantiation the dispatch below names).
 template <int DT, int TM, int TN, int EPI, int BK, int NS, int NW = 4>
 struct DmaKernelLds {
   static inline LdsKernel entry{(const void*)gemm_nt_dma_kernel<DT, TM, TN, EPI, BK, NS, NW>, NS * (2 * TM * 32 + (NW / 2) * TN * 32) * BK * 2};
+};
+template <int DT, int EPI>
+struct StreamKernelLds {
+  static inline LdsKernel entry{(const void*)gemm_stream_kernel<DT, EPI>, 2 * 512 * 128};
 };
 template <int DT, int TM, int TN, int EPI>
 struct StagedKernelLds {
@@ -661,6 +828,19 @@ static hipError_t launch_gemm(GemmArgs g, hipStream_t s) {
   if constexpr (DT != kF32) if (g.K % kDmaBK == 0) {
     constexpr int kDmaLds = kDmaStages * (BM + BR) * kDmaBK * 2;
     static_assert(kDmaLds <= 160 * 1024, "LDS ring exceeds 160 KiB");
+    if constexpr (TM == 4 && TN == 4 && (EPI == kEpiPlain || EPI == kEpiSwiglu || EPI == kEpiResidual)) {
+      // full tiles in whole rounds of 256, K tiles enough for the two-stage prologue, nothing meant to run beside it: one
+      // block per CU streams through its tiles (buffer loads: operands below 1 Gi elements, 16-byte aligned)
+      const bool covers = g.exclusive && g.M % BM == 0 && g.N % BN == 0 && g.K >= 2 * kDmaBK && blocks % 256 == 0 && g.wide &&
+                          !g.save_gate && !(EPI != kEpiSwiglu && g.b1) && (int64_t)g.M * g.K < (1ll << 30) &&
+                          (int64_t)g.N * g.K < (1ll << 30) && (uintptr_t)g.a % 16 == 0 && (uintptr_t)g.b0 % 16 == 0 &&
+                          (EPI != kEpiSwiglu || (uintptr_t)g.b1 % 16 == 0);
+      if (covers) {
+        if (hipError_t e = StreamKernelLds<DT, EPI>::entry.ensure(); e != hipSuccess) return e;
+        hipLaunchKernelGGL((gemm_stream_kernel<DT, EPI>), dim3(256), dim3(512), 2 * 512 * 128, s, g);
+        return hipGetLastError();
+      }
+    }
     if constexpr (TM == 4 && TN == 4) {
       // the 256 x 256 block tile on 8 waves of 128 x 64, two per SIMD: one wave's barrier and load waits are the other's
       // issue slots (gate/up projection at 4096 x 4096 x 1024: 66.7 against 69.1 us), at 6 fragment reads per 8 MFMAs
@@ -694,12 +874,13 @@ static int to_code(hipError_t e) { return e == hipSuccess ? OMNI_OK : OMNI_ERR_H
 // C[M,N] = A[M,K] B[N,K]^T (+ res), picking the tile shape from the problem size.
 template <int DT>
 static int gemm_plain(const void* a, const void* b, const void* b_hi, const void* res, void* c, int64_t M, int64_t N, int64_t K, hipStream_t s,
-                      float* part_mean = nullptr, float* part_m2 = nullptr) {
+                      float* part_mean = nullptr, float* part_m2 = nullptr, bool exclusive = true) {
   if (int e = check_gemm(M, N, K, ElemBytes<DT>::value)) return e;
   if (M == 0) return OMNI_OK;
   GemmArgs g{(const uint8_t*)a, (const uint8_t*)b, (const uint8_t*)b_hi, (const uint8_t*)res, (uint8_t*)c, (int)M, (int)N, (int)K, 0, 0, 0, 0, 0, 0, nullptr, nullptr, nullptr};
   g.part_mean = part_mean;
   g.part_m2 = part_m2;
+  g.exclusive = exclusive;
   const int64_t big = ((M + 255) / 256) * ((N + 255) / 256), mid = ((M + 127) / 128) * ((N + 127) / 128);
   hipError_t err;
   if (res) {
@@ -720,11 +901,12 @@ static int gemm_plain(const void* a, const void* b, const void* b_hi, const void
 
 template <int DT>
 static int gemm_swiglu(const void* x, const void* wg, const void* wu, void* h, int64_t M, int64_t I, int64_t K, hipStream_t s,
-                       void* save_gate = nullptr, void* save_up = nullptr) {
+                       void* save_gate = nullptr, void* save_up = nullptr, bool exclusive = true) {
   if (int e = check_gemm(M, I, K, ElemBytes<DT>::value)) return e;
   if (M == 0) return OMNI_OK;
   GemmArgs g{(const uint8_t*)x, (const uint8_t*)wg, (const uint8_t*)wu, nullptr, (uint8_t*)h, (int)M, (int)I, (int)K, 0, 0, 0, 0, 0, 0, nullptr, nullptr, nullptr,
              (uint8_t*)save_gate, (uint8_t*)save_up};
+  g.exclusive = exclusive;
   if (save_gate) {   // the saving epilogue has the 16-byte form only, in the direct-to-LDS kernel
     if (DT == kF32 || I % 8 != 0 || K % 64 != 0 || (uintptr_t)h % 16 || (uintptr_t)save_gate % 16 || (uintptr_t)save_up % 16) return OMNI_ERR_UNSUPPORTED;
   }
@@ -805,19 +987,39 @@ extern "C" OMNI_API int32_t omni_mlp_fwd(const void* x, const void* gate_weight,
   }
 }
 
-extern "C" OMNI_API int32_t omni_swiglu_linear_fwd(const void* x, const void* gate_weight, const void* up_weight, void* h,
-                                                   int64_t num_tokens, int32_t hidden_size, int32_t intermediate_size,
-                                                   int32_t dtype, void* stream) {
-  using namespace omni;
+// The two projection calls with the caller's word on whether anything runs beside them (the whole-layer call on two
+// streams says no to `exclusive`, which keeps the GEMMs off the streaming form that would hold every CU).
+namespace omni {
+int swiglu_linear_fwd_impl(const void* x, const void* gate_weight, const void* up_weight, void* h, int64_t num_tokens,
+                           int32_t hidden_size, int32_t intermediate_size, int32_t dtype, void* stream, bool exclusive) {
   if (num_tokens == 0) return OMNI_OK;
   if (!x || !gate_weight || !up_weight || !h) return OMNI_ERR_NULL;
   hipStream_t s = (hipStream_t)stream;
   switch (dtype) {
-    case OMNI_BF16: return gemm_swiglu<kBF16>(x, gate_weight, up_weight, h, num_tokens, intermediate_size, hidden_size, s);
-    case OMNI_F16: return gemm_swiglu<kF16>(x, gate_weight, up_weight, h, num_tokens, intermediate_size, hidden_size, s);
-    case OMNI_F32: return gemm_swiglu<kF32>(x, gate_weight, up_weight, h, num_tokens, intermediate_size, hidden_size, s);
+    case OMNI_BF16: return gemm_swiglu<kBF16>(x, gate_weight, up_weight, h, num_tokens, intermediate_size, hidden_size, s, nullptr, nullptr, exclusive);
+    case OMNI_F16: return gemm_swiglu<kF16>(x, gate_weight, up_weight, h, num_tokens, intermediate_size, hidden_size, s, nullptr, nullptr, exclusive);
+    case OMNI_F32: return gemm_swiglu<kF32>(x, gate_weight, up_weight, h, num_tokens, intermediate_size, hidden_size, s, nullptr, nullptr, exclusive);
     default: return OMNI_ERR_DTYPE;
   }
+}
+int linear_fwd_impl(const void* x, const void* weight, const void* residual, void* y, int64_t num_tokens, int32_t in_features,
+                    int32_t out_features, int32_t dtype, void* stream, bool exclusive) {
+  if (num_tokens == 0) return OMNI_OK;
+  if (!x || !weight || !y) return OMNI_ERR_NULL;
+  hipStream_t s = (hipStream_t)stream;
+  switch (dtype) {
+    case OMNI_BF16: return gemm_plain<kBF16>(x, weight, nullptr, residual, y, num_tokens, out_features, in_features, s, nullptr, nullptr, exclusive);
+    case OMNI_F16: return gemm_plain<kF16>(x, weight, nullptr, residual, y, num_tokens, out_features, in_features, s, nullptr, nullptr, exclusive);
+    case OMNI_F32: return gemm_plain<kF32>(x, weight, nullptr, residual, y, num_tokens, out_features, in_features, s, nullptr, nullptr, exclusive);
+    default: return OMNI_ERR_DTYPE;
+  }
+}
+}  // namespace omni
+
+extern "C" OMNI_API int32_t omni_swiglu_linear_fwd(const void* x, const void* gate_weight, const void* up_weight, void* h,
+                                                   int64_t num_tokens, int32_t hidden_size, int32_t intermediate_size,
+                                                   int32_t dtype, void* stream) {
+  return omni::swiglu_linear_fwd_impl(x, gate_weight, up_weight, h, num_tokens, hidden_size, intermediate_size, dtype, stream, true);
 }
 
 extern "C" OMNI_API int32_t omni_swiglu_linear_save_fwd(const void* x, const void* gate_weight, const void* up_weight, void* h,
@@ -837,16 +1039,7 @@ extern "C" OMNI_API int32_t omni_swiglu_linear_save_fwd(const void* x, const voi
 
 extern "C" OMNI_API int32_t omni_linear_fwd(const void* x, const void* weight, const void* residual, void* y, int64_t num_tokens,
                                             int32_t in_features, int32_t out_features, int32_t dtype, void* stream) {
-  using namespace omni;
-  if (num_tokens == 0) return OMNI_OK;
-  if (!x || !weight || !y) return OMNI_ERR_NULL;
-  hipStream_t s = (hipStream_t)stream;
-  switch (dtype) {
-    case OMNI_BF16: return gemm_plain<kBF16>(x, weight, nullptr, residual, y, num_tokens, out_features, in_features, s);
-    case OMNI_F16: return gemm_plain<kF16>(x, weight, nullptr, residual, y, num_tokens, out_features, in_features, s);
-    case OMNI_F32: return gemm_plain<kF32>(x, weight, nullptr, residual, y, num_tokens, out_features, in_features, s);
-    default: return OMNI_ERR_DTYPE;
-  }
+  return omni::linear_fwd_impl(x, weight, residual, y, num_tokens, in_features, out_features, dtype, stream, true);
 }
 
 extern "C" OMNI_API int32_t omni_linear2_fwd(const void* x, const void* weight_lo, const void* weight_hi, void* y,
