@@ -45,10 +45,11 @@ HBM_PEAK_GBS = 8000.0           # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 # Bytes that cross the fabric per launch (FETCH_SIZE + WRITE_SIZE of rocprofv3 --pmc, each scaled by a plain copy of
 # known size); counters cannot be read in-process, so these are the figures of the committed summaries named here.
-TRAFFIC_SOURCE = "profiles/bench_layer_c4_hbm_counters.txt, profiles/expert_c5_hbm_counters.txt"
-TRAFFIC_BYTES = {"expert_c3": 180.6e6, "expert_c4": 57.8e6, "expert_gather_c3": 897.2e6, "gateup_c4": 134.4e6, "down_c4": 117.6e6,
-                 "down_plain_c4": 109.2e6, "schedule_c3": 12.36e6,
-                 "expert_c5_routed": 1029.2e6, "expert_c5_uniform": 8846.8e6}
+TRAFFIC_SOURCE = ("profiles/bench_layer_c4_hbm_counters.txt, profiles/expert_c5_hbm_counters.txt; measured on the kernels as of the commit "
+                  "'GEMM: streaming form of the 256x256 tile' -- a later change to a kernel's memory access pattern needs a new counter run")
+TRAFFIC_BYTES = {"expert_c3": 180.6e6, "expert_c4": 57.8e6, "expert_gather_c3": 899.4e6, "gateup_c4": 134.5e6, "down_c4": 117.6e6,
+                 "down_plain_c4": 109.2e6, "schedule_c3": 12.36e6, "expert_segment_c3": 928.2e6, "expert_bwd_c3": 2159.4e6,
+                 "expert_c5_routed": 1029.2e6, "expert_c5_routed_split": 724.7e6, "expert_c5_uniform": 8846.8e6}
 SECTIONS = ("layer", "kernels", "expert_c3", "expert_c5", "layer_c5", "ref_grid", "probe", "train", "cpu")
 
 
@@ -270,8 +271,14 @@ def main():
         h = hip.hip_swiglu_linear_func(xf, layer.gate_proj.weight, layer.up_proj.weight)
         y0 = hip.hip_linear_func(h, layer.down_proj.weight)
         r = layer.num_expert_sqrt
-        m, b = time_launches(torch, lambda: hip.hip_swiglu_linear_func(xf, layer.gate_proj.weight, layer.up_proj.weight))
-        kernels.append(mfma_entry("gemm_nt_dma_kernel<swiglu> (gate/up projection + SwiGLU), c4", 4 * T * H * I, m, b, TRAFFIC_BYTES["gateup_c4"], sustained))
+        # the gate/up projection as the two-stream layer step runs it (a grid of 512 blocks that leaves room for the side branch) ...
+        m, b = time_launches(torch, lambda: hip.hip_swiglu_linear_func(xf, layer.gate_proj.weight, layer.up_proj.weight, shared=True))
+        kernels.append(mfma_entry("gemm_nt_dma_kernel<swiglu> (gate/up projection + SwiGLU, as in the two-stream layer step), c4", 4 * T * H * I, m, b, TRAFFIC_BYTES["gateup_c4"], sustained))
+        # ... and as every caller gets it that has the GPU to itself (operator calls, the one-stream layer): one block per CU streaming through its tiles
+        m_s, b_s = time_launches(torch, lambda: hip.hip_swiglu_linear_func(xf, layer.gate_proj.weight, layer.up_proj.weight))
+        kernels[-1]["streaming_form_alone_ms"] = m_s
+        kernels[-1]["streaming_form_alone_ms_best"] = b_s
+        kernels[-1]["streaming_form_frac"] = 4 * T * H * I / (m_s * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS
         # for orientation: the vendor library (torch.matmul) on the same operands, without the SwiGLU (one GEMM over [Wg; Wu])
         wcat = torch.cat([layer.gate_proj.weight, layer.up_proj.weight], 0)
         m_lib, b_lib = time_launches(torch, lambda: torch.matmul(xf, wcat.t()))
@@ -290,9 +297,14 @@ def main():
         kernels.append(hbm_entry("expert op (split algorithm: expert_split_dots_kernel + expert_split_accumulate_kernel), c4", m, b,
                                  expert_alg_bytes(T, H, k), TRAFFIC_BYTES["expert_c4"], expert_min_bytes(T, H, N, k)))
         m, b = time_launches(torch, lambda: layer.route(xf))
+        layer.eval()
+        m_e, b_e = time_launches(torch, lambda: layer.route(xf))
+        layer.train()
         kernels.append({"kernel": "router stage (projection GEMM with BN statistics epilogue + BN finalize + select), c4", "kernel_ms": m,
-                        "kernel_ms_best": b, "algorithmic_flops": 4 * T * H * r, "algorithmic_bytes": (T * H + 2 * r * H + T * k * 3) * 2,
-                        "note": "1.07 GFLOP over 9.7 MB: bounded by launch and memory latency, not by a roofline"})
+                        "kernel_ms_best": b, "eval_mode_ms": m_e, "eval_mode_ms_best": b_e,
+                        "algorithmic_flops": 4 * T * H * r, "algorithmic_bytes": (T * H + 2 * r * H + T * k * 3) * 2,
+                        "note": "1.07 GFLOP over 9.7 MB: bounded by launch and memory latency, not by a roofline; training = three dependent "
+                                "launches, eval = two (the select kernel reads the running statistics itself)"})
         out["roofline"] = kernels[0]
 
     if "expert_c3" in sections:
@@ -321,7 +333,8 @@ def main():
                                  note="ids in, pair ids + token ids + offsets out; writes equal the algorithmic 2.1 MB (every output line goes through one L2), the ids are fetched by all 8 XCDs"))
         m, b = time_launches(torch, lambda: hip.hip_omni_expert_func(x3, up3, down3, g3, i3, algo="segment"))
         kernels.append(hbm_entry("expert op, expert-centric 'segment' algorithm (schedule + scores pass + token pass), c3", m, b,
-                                 expert_alg_bytes(T3, H, k), note="for comparison; same results as the gather algorithm"))
+                                 expert_alg_bytes(T3, H, k), TRAFFIC_BYTES["expert_segment_c3"], expert_min_bytes(T3, H, N, k),
+                                 note="for comparison; same results as the gather algorithm"))
         # the reference's group regime (omni_scheduler.py:58: tokens x k / experts > 256): same tokens, 256 experts; AUTO takes
         # the dense algorithm (two MFMA GEMMs over all experts), timed beside the gather algorithm on the same inputs
         Ng = 256
@@ -330,7 +343,7 @@ def main():
         yg = hip.hip_omni_expert_func(xg, upg, downg, gg, ig, algo="dense")
         wantg = oracle.expert_forward(xg_c[:sub], upg_c, downg_c, gg_c[:sub], ig_c[:sub])
         torch.testing.assert_close(yg[:sub].float().cpu(), wantg.float(), rtol=2e-2, atol=2e-2)
-        m, b = time_launches(torch, lambda: hip.hip_omni_expert_func(xg, upg, downg, gg, ig))
+        m, b = time_launches(torch, lambda: hip.hip_omni_expert_func(xg, upg, downg, gg, ig, algo="dense"))
         dense = mfma_entry("expert op, dense algorithm (gate rows + transpose + two MFMA GEMMs), group regime: 16384 tokens, 256 experts, top-16",
                            2 * T3 * H * Ng + 2 * T3 * H * 2 * Ng, m, b, None, None)
         m, b = time_launches(torch, lambda: hip.hip_omni_expert_func(xg, upg, downg, gg, ig, algo="gather"))
@@ -344,7 +357,7 @@ def main():
             dy3 = x3 * 0.5
             m, b = time_launches(torch, lambda: hip.hip_omni_expert_bwd_func(dy3, x3, up3, down3, g3, i3), n=10)
             kernels.append(hbm_entry("expert op backward (schedule + token pass + weight pass), c3", m, b, expert_bwd_alg_bytes(T3, H, N, k),
-                                     note="x, dy (32 MiB each) and the tables are cache-resident"))
+                                     TRAFFIC_BYTES["expert_bwd_c3"], note="x, dy (32 MiB each) and the tables are cache-resident"))
         del x3, up3, down3, g3, i3, y3
 
     if "expert_c5" in sections or "layer_c5" in sections:
@@ -433,15 +446,19 @@ def main():
             m, b = time_launches(torch, lambda: layer5(x5.view(8, T5 // 8, H5)), n=5, reps=5, warmup=2)
             per_algo[algo] = {"ms_per_step": m, "ms_per_step_best": b, "tokens_per_s": T5 / (m * 1e-3)}
         layer5.expert_algo = "auto"
+        # the module's default at this size is one stream (OmniMoE.overlap_max_work); the two-stream schedule beside it
+        layer5.overlap_max_work = 2 ** 62
+        m2, b2 = time_launches(torch, lambda: layer5(x5.view(8, T5 // 8, H5)), n=5, reps=5, warmup=2)
+        del layer5.overlap_max_work
         xf5 = x5
         m_gu, b_gu = time_launches(torch, lambda: hip.hip_swiglu_linear_func(xf5, layer5.gate_proj.weight, layer5.up_proj.weight), n=5, reps=5, warmup=2)
-        e_gu = mfma_entry("gemm_nt_dma_kernel<swiglu> (gate/up projection + SwiGLU), config 5 (32768 x 2 x 8192 x 2048)", 4 * T5 * H5 * I5, m_gu, b_gu, None, sustained)
+        e_gu = mfma_entry("gemm_stream_kernel<swiglu> (gate/up projection + SwiGLU), config 5 (32768 x 2 x 8192 x 2048)", 4 * T5 * H5 * I5, m_gu, b_gu, None, sustained)
         h5 = hip.hip_swiglu_linear_func(xf5, layer5.gate_proj.weight, layer5.up_proj.weight)
         m_d, b_d = time_launches(torch, lambda: hip.hip_linear_func(h5, layer5.down_proj.weight), n=5, reps=5, warmup=2)
-        e_d = mfma_entry("gemm_nt_dma_kernel<plain> (down projection), config 5 (32768 x 2048 x 8192)", 2 * T5 * H5 * I5, m_d, b_d, None, sustained)
+        e_d = mfma_entry("gemm_stream_kernel<plain> (down projection), config 5 (32768 x 2048 x 8192)", 2 * T5 * H5 * I5, m_d, b_d, None, sustained)
         wcat5 = torch.cat([wx5, wy5], 0)
         m_r, b_r = time_launches(torch, lambda: hip.hip_linear_func(xf5, wcat5), n=5, reps=5, warmup=2)
-        e_r = mfma_entry("gemm_nt_dma_kernel<plain> (router projection, both halves: 32768 x 1024 x 2048; arithmetic intensity 669 flop/B), config 5",
+        e_r = mfma_entry("gemm_stream_kernel<plain> (router projection, both halves: 32768 x 1024 x 2048; arithmetic intensity 669 flop/B), config 5",
                          4 * T5 * H5 * r5, m_r, b_r, None, sustained)
         m_lib, _ = time_launches(torch, lambda: torch.matmul(xf5, wcat5.t()), n=5, reps=3, warmup=2)
         e_r["library_gemm_same_flops_ms"] = m_lib
@@ -456,7 +473,8 @@ def main():
         out["layer_c5"] = {"workload": "BASELINE.json configs[4] (benchmark config 5): full OmniMoE layer forward, 8x4096 tokens, hidden 2048, intermediate 8192, "
                                        "262144 experts (512x512), top-32, eval-mode BatchNorm whose buffers carry the Zipf(1.1) key bias, seed 4",
                            "ms_per_step": per_algo["auto"]["ms_per_step"], "tokens_per_s": per_algo["auto"]["tokens_per_s"],
-                           "with_expert_algo_split": per_algo["split"], "router_stage_ms": m_rt,
+                           "with_expert_algo_split": per_algo["split"], "on_two_streams": {"ms_per_step": m2, "ms_per_step_best": b2},
+                           "router_stage_ms": m_rt,
                            "gate_up_TFLOPs": e_gu["achieved"], "down_TFLOPs": e_d["achieved"], "router_projection_TFLOPs": e_r["achieved"],
                            "frac_of_mfma_peak": {"gate_up": e_gu["frac"], "down": e_d["frac"], "router_projection": e_r["frac"]},
                            "checked": f"{sub} tokens against the oracle (router ids, experts over the selected rows, MLP) before timing"}

@@ -172,6 +172,15 @@ OMNI_API int32_t omni_swiglu_linear_fwd(const void* x, const void* gate_weight, 
 OMNI_API int32_t omni_linear_fwd(const void* x, const void* weight, const void* residual, void* y, int64_t num_tokens,
                                  int32_t in_features, int32_t out_features, int32_t dtype, void* stream);
 
+/* omni_swiglu_linear_fwd for callers that run other kernels beside it (another stream).  Where the product is whole rounds
+ * of 256 x 256 tiles, omni_swiglu_linear_fwd / omni_linear_fwd / omni_mlp_fwd launch one block per CU that walks its share
+ * of the tiles -- faster alone, but it holds every CU until it ends, so a concurrent kernel waits.  This entry never takes
+ * that form (omni_moe_fwd with a side stream uses it for the gate/up projection).  Same results bit for bit.
+ * No counterpart in the reference. */
+OMNI_API int32_t omni_swiglu_linear_fwd_shared(const void* x, const void* gate_weight, const void* up_weight, void* h,
+                                               int64_t num_tokens, int32_t hidden_size, int32_t intermediate_size,
+                                               int32_t dtype, void* stream);
+
 /* omni_swiglu_linear_fwd that also keeps the two projections a backward pass needs (the reference materialises them:
  * interface.py:23-27 calls torch.matmul twice before the SwiGLU function saves gate and up, omni_mlp.py:359-371):
  *   gate_out, up_out [T,I]: x Wg^T and x Wu^T rounded to the storage dtype; h [T,I] their SwiGLU product.

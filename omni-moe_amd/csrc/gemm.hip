@@ -1022,6 +1022,12 @@ extern "C" OMNI_API int32_t omni_swiglu_linear_fwd(const void* x, const void* ga
   return omni::swiglu_linear_fwd_impl(x, gate_weight, up_weight, h, num_tokens, hidden_size, intermediate_size, dtype, stream, true);
 }
 
+extern "C" OMNI_API int32_t omni_swiglu_linear_fwd_shared(const void* x, const void* gate_weight, const void* up_weight, void* h,
+                                                          int64_t num_tokens, int32_t hidden_size, int32_t intermediate_size,
+                                                          int32_t dtype, void* stream) {
+  return omni::swiglu_linear_fwd_impl(x, gate_weight, up_weight, h, num_tokens, hidden_size, intermediate_size, dtype, stream, false);
+}
+
 extern "C" OMNI_API int32_t omni_swiglu_linear_save_fwd(const void* x, const void* gate_weight, const void* up_weight, void* h,
                                                         void* gate_out, void* up_out, int64_t num_tokens, int32_t hidden_size,
                                                         int32_t intermediate_size, int32_t dtype, void* stream) {

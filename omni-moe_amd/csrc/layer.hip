@@ -11,10 +11,8 @@ static inline size_t up256(size_t v) { return (v + 255) / 256 * 256; }
 static inline size_t elem_bytes(int dtype) { return dtype == OMNI_F32 ? 4 : 2; }
 // defined beside the expert kernels: OMNI_OK when omni_expert_fwd takes `algo` at this shape (decided from the sizes alone)
 int expert_algo_check(int algo, int64_t num_tokens, int hidden_size, int64_t num_experts, int top_k, int dtype);
-// defined beside the GEMM kernels: omni_swiglu_linear_fwd / omni_linear_fwd with the caller's word on whether the launch has
-// the GPU to itself (then a GEMM of whole 256-tile rounds may take the form that holds every CU until it ends)
-int swiglu_linear_fwd_impl(const void* x, const void* gate_weight, const void* up_weight, void* h, int64_t num_tokens,
-                           int32_t hidden_size, int32_t intermediate_size, int32_t dtype, void* stream, bool exclusive);
+// defined beside the GEMM kernels: omni_linear_fwd with the caller's word on whether the launch has the GPU to itself
+// (then a GEMM of whole 256-tile rounds may take the form that holds every CU until it ends)
 int linear_fwd_impl(const void* x, const void* weight, const void* residual, void* y, int64_t num_tokens, int32_t in_features,
                     int32_t out_features, int32_t dtype, void* stream, bool exclusive);
 }  // namespace omni
@@ -104,7 +102,8 @@ extern "C" OMNI_API int32_t omni_moe_fwd_algo(const void* x, const void* gate_we
                           running_mean_y, running_var_y, num_batches_tracked_y, training, momentum, eps, gates, ids, nullptr,
                           num_tokens, hidden_size, num_expert_sqrt, num_experts_per_token, dtype, stats_dtype, router_ws, branch);
   const bool alone = side_stream == nullptr;            // one stream: every kernel runs by itself
-  if (!e) e = swiglu_linear_fwd_impl(x, gate_weight, up_weight, h, num_tokens, hidden_size, intermediate_size, dtype, main_s, alone);
+  if (!e) e = alone ? omni_swiglu_linear_fwd(x, gate_weight, up_weight, h, num_tokens, hidden_size, intermediate_size, dtype, main_s)
+                    : omni_swiglu_linear_fwd_shared(x, gate_weight, up_weight, h, num_tokens, hidden_size, intermediate_size, dtype, main_s);
   if (!e) e = omni_expert_fwd(x, up_embed, down_embed, gates, ids, experts, num_tokens, hidden_size, num_experts,
                               num_experts_per_token, dtype, expert_algo, expert_ws, branch);
   if (!side_stream) {   // one stream: the add is the down projection's epilogue

@@ -98,6 +98,12 @@ class OmniMoE(nn.Module):
     # The fork and join cost about 50 us of host time per call, so below this much work (tokens x hidden x
     # intermediate; 2048 x 1024 x 4096 measured level on an MI355X) the call would be host-bound: one stream then.
     overlap_min_work = 2 ** 33
+    # ... and from this much work on, one stream is the faster schedule again: alone on the GPU the two big GEMMs take their
+    # streaming form (one block per CU walking its output tiles), which beats what the side branch gains beside them -- the
+    # chip is power-limited under the GEMMs, so overlapped kernels slow each other by about what they would cost alone
+    # (measured, hidden 1024 x intermediate 4096: 4096 tokens 134 against 143 us on two streams, 8192 tokens equal,
+    # 65536 tokens 1.85 against 1.70 ms; benchmark config 5: 3.58 against 3.43 ms).
+    overlap_max_work = 2 ** 35
     # Expert algorithm of the fused forward: "auto" decides from the sizes alone (no device-to-host read).  Which one is
     # faster also depends on how many DISTINCT experts the router picks: with tables far beyond the caches and a skewed
     # router (few live experts) "split" beats auto's "gather"; the caller who knows the distribution says so here.
@@ -136,8 +142,8 @@ class OmniMoE(nn.Module):
         nx, ny = self._router_norms()
         with torch.no_grad():
             x = hidden_states.view(-1, self.hidden_size)
-            two = (self.overlap_branches and x.is_cuda
-                   and x.size(0) * self.hidden_size * self.intermediate_size > self.overlap_min_work)
+            work = x.size(0) * self.hidden_size * self.intermediate_size
+            two = self.overlap_branches and x.is_cuda and self.overlap_min_work < work < self.overlap_max_work
             side, fork, join = self._branch_resources(x.device) if two else (None, None, None)
             out = hip_omni_moe_fwd_func(
                 x, self.gate_proj.weight, self.up_proj.weight, self.down_proj.weight,

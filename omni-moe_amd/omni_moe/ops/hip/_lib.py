@@ -36,6 +36,7 @@ SIGNATURES = {
     "omni_mlp_fwd": (c_int32, [c_void_p] * 6 + [c_int64, c_int32, c_int32, c_int32, c_void_p, c_void_p]),
     "omni_linear_fwd": (c_int32, [c_void_p] * 4 + [c_int64, c_int32, c_int32, c_int32, c_void_p]),
     "omni_swiglu_linear_fwd": (c_int32, [c_void_p] * 4 + [c_int64, c_int32, c_int32, c_int32, c_void_p]),
+    "omni_swiglu_linear_fwd_shared": (c_int32, [c_void_p] * 4 + [c_int64, c_int32, c_int32, c_int32, c_void_p]),
     "omni_swiglu_linear_save_fwd": (c_int32, [c_void_p] * 6 + [c_int64, c_int32, c_int32, c_int32, c_void_p]),
     "omni_moe_workspace_bytes": (c_size_t, [c_int64, c_int32, c_int32, c_int64, c_int32, c_int32, c_int32]),
     "omni_moe_fwd": (c_int32, [c_void_p] * 15 + [c_int64, c_int32, c_int32, c_int64, c_int32, c_int32, c_int32, c_int32,

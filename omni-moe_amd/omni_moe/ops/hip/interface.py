@@ -410,8 +410,9 @@ class OmniSwiGLUFunc(torch.autograd.Function):
         return hip_swiglu_bwd_func(dout, gate, up)
 
 
-def hip_swiglu_linear_func(x: torch.Tensor, gate_weight: torch.Tensor, up_weight: torch.Tensor) -> torch.Tensor:
-    """silu(x gate^T) * (x up^T): the first half of the MLP op as one GEMM with a fused epilogue."""
+def hip_swiglu_linear_func(x: torch.Tensor, gate_weight: torch.Tensor, up_weight: torch.Tensor, shared: bool = False) -> torch.Tensor:
+    """silu(x gate^T) * (x up^T): the first half of the MLP op as one GEMM with a fused epilogue.  ``shared=True`` says that
+    other kernels run beside it (another stream): the launch then never takes the form that holds every CU."""
     if x.dim() != 2 or gate_weight.shape != up_weight.shape or gate_weight.dim() != 2 or gate_weight.size(1) != x.size(1):
         raise ValueError("expected x (tokens, hidden) and gate/up weights (intermediate, hidden)")
     if x.dtype not in _lib.DTYPE_CODE or gate_weight.dtype != x.dtype or up_weight.dtype != x.dtype:
@@ -420,9 +421,9 @@ def hip_swiglu_linear_func(x: torch.Tensor, gate_weight: torch.Tensor, up_weight
     x, gate_weight, up_weight = map(_c, (x, gate_weight, up_weight))
     h = torch.empty((x.size(0), gate_weight.size(0)), device=dev, dtype=x.dtype)
     with torch.cuda.device(dev):
-        code = _lib.load().omni_swiglu_linear_fwd(_lib.ptr(x), _lib.ptr(gate_weight), _lib.ptr(up_weight), _lib.ptr(h),
-                                                  x.size(0), x.size(1), gate_weight.size(0), _lib.DTYPE_CODE[x.dtype],
-                                                  _lib.stream_ptr())
+        fn = _lib.load().omni_swiglu_linear_fwd_shared if shared else _lib.load().omni_swiglu_linear_fwd
+        code = fn(_lib.ptr(x), _lib.ptr(gate_weight), _lib.ptr(up_weight), _lib.ptr(h), x.size(0), x.size(1), gate_weight.size(0),
+                  _lib.DTYPE_CODE[x.dtype], _lib.stream_ptr())
     _lib.check(code, "omni_swiglu_linear_fwd")
     return h
 
