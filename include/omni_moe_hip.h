@@ -120,9 +120,11 @@ OMNI_API int32_t omni_schedule_noalloc(const int32_t* indices, int32_t* offsets,
  *   algo      : OMNI_EXPERT_ALGO_*.  GATHER: one wave per token fetches whole rows.  SPLIT: the hidden
  *               dimension in 8 slices, slice s handled by the blocks that run on XCD s, so that
  *               each XCD's L2 holds its eighth of both tables; two launches and [8][T][k] floats
- *               of partial dot products (H*sizeof(elem)/8 must be 64..1024 bytes, a power of two).
+ *               of partial dot products (H*sizeof(elem)/8 must be 64..1024 bytes, a power of two; wider rows are
+ *               taken in up to 64 column blocks of that form, one pair of launches per block, [8 * blocks][T][k] floats).
+ *               Rows beyond 8 KiB exist for SPLIT only, and AUTO is SPLIT for them.
  *               AUTO = SPLIT when the tables overflow one L2 but an eighth of them fits and there
- *               are >= 32768 pairs, else GATHER.  SEGMENT is the expert-centric organisation:
+ *               are >= 32768 pairs (and for rows beyond 8 KiB), else GATHER.  SEGMENT is the expert-centric organisation:
  *               omni_schedule, a pass over the sorted pairs for the coefficients, a token pass
  *               for the sum; kept so that the organisations can be measured side by side.
  *               GATHER and SEGMENT agree bit for bit, SPLIT to fp32 rounding of the dot products.

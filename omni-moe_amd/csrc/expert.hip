@@ -312,7 +312,7 @@ __device__ __forceinline__ float reduce_scatter_group(float (&v)[N], const int l
 template <int DT, int LPR>
 __global__ __launch_bounds__(kTokensPerBlock* kWave) void expert_split_dots_kernel(
     const uint8_t* __restrict__ x, const uint8_t* __restrict__ up, const int32_t* __restrict__ ids,
-    float* __restrict__ partial, int num_tokens, int hidden, int top_k, uint32_t num_experts) {
+    float* __restrict__ partial, int num_tokens, int hidden, int top_k, uint32_t num_experts, int col_block) {
   constexpr int E = Row16<DT>::kElems, GP = kWave / LPR;
   constexpr int LD = LPR < 8 ? LPR : 8;                          // row loads in flight at a time
   const int lane = lane_id(), sub = lane % LPR, grp = lane / LPR;
@@ -321,7 +321,8 @@ __global__ __launch_bounds__(kTokensPerBlock* kWave) void expert_split_dots_kern
   const bool live = t < num_tokens;
   const int tt = live ? t : 0;
   const int64_t row_bytes = int64_t(hidden) * (16 / E);
-  const int64_t col = int64_t(slice) * LPR * 16 + sub * 16;      // this lane's 16 bytes inside a row
+  // this lane's 16 bytes inside a row (rows wider than 8 slices of 64 lanes go in column blocks of 8 slices, one launch each)
+  const int64_t col = (int64_t(col_block) * kSlices + slice) * LPR * 16 + sub * 16;
   const u32x4_t xr = *(const u32x4_t*)(x + tt * row_bytes + col);
   const int64_t base = int64_t(tt) * top_k;
   for (int jb = 0; jb < top_k; jb += LPR) {
@@ -343,7 +344,7 @@ __global__ __launch_bounds__(kTokensPerBlock* kWave) void expert_split_dots_kern
     const int j = jb + sub;
     if (live && j < top_k) {
       const bool ok = (uint32_t)my_id < num_experts;
-      partial[(int64_t(slice) * num_tokens + t) * top_k + j] = ok ? total : 0.f;
+      partial[((int64_t(col_block) * kSlices + slice) * num_tokens + t) * top_k + j] = ok ? total : 0.f;
     }
   }
 }
@@ -354,7 +355,8 @@ __global__ __launch_bounds__(kTokensPerBlock* kWave) void expert_split_dots_kern
 template <int DT, int LPR>
 __global__ __launch_bounds__(kTokensPerBlock* kWave) void expert_split_accumulate_kernel(
     const uint8_t* __restrict__ down, const void* __restrict__ gates, const int32_t* __restrict__ ids,
-    const float* __restrict__ partial, uint8_t* __restrict__ y, int num_tokens, int hidden, int top_k, uint32_t num_experts) {
+    const float* __restrict__ partial, uint8_t* __restrict__ y, int num_tokens, int hidden, int top_k, uint32_t num_experts,
+    int col_block, int col_blocks) {
   constexpr int E = Row16<DT>::kElems, GP = kWave / LPR;
   constexpr int LD = LPR < 8 ? LPR : 8;
   const int lane = lane_id(), sub = lane % LPR, grp = lane / LPR;
@@ -363,7 +365,7 @@ __global__ __launch_bounds__(kTokensPerBlock* kWave) void expert_split_accumulat
   const bool live = t < num_tokens;
   const int tt = live ? t : 0;
   const int64_t row_bytes = int64_t(hidden) * (16 / E);
-  const int64_t col = int64_t(slice) * LPR * 16 + sub * 16;
+  const int64_t col = (int64_t(col_block) * kSlices + slice) * LPR * 16 + sub * 16;
   const int64_t base = int64_t(tt) * top_k;
   float acc[E];
 #pragma unroll
@@ -389,8 +391,10 @@ __global__ __launch_bounds__(kTokensPerBlock* kWave) void expert_split_accumulat
     float coef = 0.f;
     if (my_id >= 0) {
       float sdot = 0.f;
+      for (int cb = 0; cb < col_blocks; ++cb) {                  // slice order, column block by column block
 #pragma unroll
-      for (int sl = 0; sl < kSlices; ++sl) sdot += partial[(int64_t(sl) * num_tokens + tt) * top_k + j];
+        for (int sl = 0; sl < kSlices; ++sl) sdot += partial[((int64_t(cb) * kSlices + sl) * num_tokens + tt) * top_k + j];
+      }
       coef = silu_f32(sdot) * Elem<DT>::load(gates, base + j);
     }
 #pragma unroll
@@ -410,35 +414,49 @@ static inline int split_lanes_per_row(int hidden, int elem_bytes) {
   const int lpr = (int)(slice_bytes / 16);
   return (lpr == 4 || lpr == 8 || lpr == 16 || lpr == 32 || lpr == 64) ? lpr : 0;
 }
+// Rows beyond 8 KiB (8 slices of 64 lanes): the smallest number of column blocks, each 8 slices of a power-of-two number of
+// lanes, that the row cuts into; 0 if there is none (up to 64 blocks: rows of 512 KiB).  1 for rows that split_lanes_per_row takes.
+constexpr int kMaxColBlocks = 64;
+static inline int split_col_blocks(int hidden, int elem_bytes, int* lanes_per_row) {
+  for (int b = 1; b <= kMaxColBlocks; ++b) {
+    if (hidden % b != 0) continue;
+    const int lpr = split_lanes_per_row(hidden / b, elem_bytes);
+    if (lpr) { *lanes_per_row = lpr; return b; }
+  }
+  return 0;
+}
 
 template <int DT, int LPR>
 static hipError_t launch_split(const void* x, const void* up, const void* down, const void* gates, const int32_t* ids,
-                               float* partial, void* y, int64_t T, int H, int k, int64_t N, hipStream_t s) {
+                               float* partial, void* y, int64_t T, int H, int k, int64_t N, int col_blocks, hipStream_t s) {
   constexpr int kPerBlock = kTokensPerBlock * (kWave / LPR);       // tokens per block
   const unsigned blocks = (unsigned)((T + kPerBlock - 1) / kPerBlock) * kSlices;
-  hipLaunchKernelGGL((expert_split_dots_kernel<DT, LPR>), dim3(blocks), dim3(kTokensPerBlock * kWave), 0, s, (const uint8_t*)x,
-                     (const uint8_t*)up, ids, partial, (int)T, H, k, (uint32_t)N);
-  hipLaunchKernelGGL((expert_split_accumulate_kernel<DT, LPR>), dim3(blocks), dim3(kTokensPerBlock * kWave), 0, s,
-                     (const uint8_t*)down, gates, ids, partial, (uint8_t*)y, (int)T, H, k, (uint32_t)N);
+  for (int cb = 0; cb < col_blocks; ++cb)                            // all partial dot products first: a coefficient needs the whole row
+    hipLaunchKernelGGL((expert_split_dots_kernel<DT, LPR>), dim3(blocks), dim3(kTokensPerBlock * kWave), 0, s, (const uint8_t*)x,
+                       (const uint8_t*)up, ids, partial, (int)T, H, k, (uint32_t)N, cb);
+  for (int cb = 0; cb < col_blocks; ++cb)
+    hipLaunchKernelGGL((expert_split_accumulate_kernel<DT, LPR>), dim3(blocks), dim3(kTokensPerBlock * kWave), 0, s,
+                       (const uint8_t*)down, gates, ids, partial, (uint8_t*)y, (int)T, H, k, (uint32_t)N, cb, col_blocks);
   return hipGetLastError();
 }
 
-// workspace: partial dot products [8][T][k] f32
+// workspace: partial dot products [8 * column blocks][T][k] f32
 template <int DT>
 static int expert_split_dispatch(const void* x, const void* up, const void* down, const void* gates, const int32_t* ids,
                                  void* y, int64_t T, int H, int k, int64_t N, void* workspace, hipStream_t s) {
-  const int lpr = split_lanes_per_row(H, DT == kF32 ? 4 : 2);
-  if (lpr == 0 || k > 2 * kWave) return OMNI_ERR_UNSUPPORTED;
+  int lpr = 0;
+  const int col_blocks = split_col_blocks(H, DT == kF32 ? 4 : 2, &lpr);
+  if (col_blocks == 0 || k > 2 * kWave) return OMNI_ERR_UNSUPPORTED;
   if (T == 0) return OMNI_OK;
   if (k == 0) return expert_gather_dispatch<DT>(x, up, down, gates, ids, y, T, H, k, N, s);   // writes zeros
   if (!workspace) return OMNI_ERR_WORKSPACE;
   float* partial = (float*)workspace;
   hipError_t err;
-  if (lpr == 4) err = launch_split<DT, 4>(x, up, down, gates, ids, partial, y, T, H, k, N, s);
-  else if (lpr == 8) err = launch_split<DT, 8>(x, up, down, gates, ids, partial, y, T, H, k, N, s);
-  else if (lpr == 16) err = launch_split<DT, 16>(x, up, down, gates, ids, partial, y, T, H, k, N, s);
-  else if (lpr == 32) err = launch_split<DT, 32>(x, up, down, gates, ids, partial, y, T, H, k, N, s);
-  else err = launch_split<DT, 64>(x, up, down, gates, ids, partial, y, T, H, k, N, s);
+  if (lpr == 4) err = launch_split<DT, 4>(x, up, down, gates, ids, partial, y, T, H, k, N, col_blocks, s);
+  else if (lpr == 8) err = launch_split<DT, 8>(x, up, down, gates, ids, partial, y, T, H, k, N, col_blocks, s);
+  else if (lpr == 16) err = launch_split<DT, 16>(x, up, down, gates, ids, partial, y, T, H, k, N, col_blocks, s);
+  else if (lpr == 32) err = launch_split<DT, 32>(x, up, down, gates, ids, partial, y, T, H, k, N, col_blocks, s);
+  else err = launch_split<DT, 64>(x, up, down, gates, ids, partial, y, T, H, k, N, col_blocks, s);
   return err == hipSuccess ? OMNI_OK : OMNI_ERR_HIP_BASE + (int)err;
 }
 
@@ -533,6 +551,8 @@ static int resolve_algo(int algo, int64_t T, int H, int64_t N, int k, int dtype)
   // only ever touch selected rows; and where it wins at all it wins little (the reference's group regime, T*k/N > 256
   // with N <= 16 k: 63 us against 67.5 us gather at 16384 tokens, hidden 1024, N = 256, k = 16; 95 against 70 at N = 512).
   const int es = dtype == OMNI_F32 ? 4 : 2;
+  // rows beyond 8 KiB do not fit the gather kernel's registers: the split kernels take them in column blocks
+  if ((int64_t)H * es > 8192) return OMNI_EXPERT_ALGO_SPLIT;
   const int64_t tables = 2 * N * (int64_t)H * es;
   const bool fits = split_lanes_per_row(H, es) != 0 && k <= 2 * kWave;
   if (fits && tables > (3ll << 20) && tables / kSlices <= (3ll << 20) && T * (int64_t)k >= 32768) return OMNI_EXPERT_ALGO_SPLIT;
@@ -543,8 +563,14 @@ static int resolve_algo(int algo, int64_t T, int H, int64_t N, int k, int dtype)
 int expert_algo_check(int algo, int64_t T, int H, int64_t N, int k, int dtype) {
   const int es = dtype == OMNI_F32 ? 4 : 2;
   switch (algo) {
-    case OMNI_EXPERT_ALGO_AUTO: case OMNI_EXPERT_ALGO_GATHER: case OMNI_EXPERT_ALGO_SEGMENT: return OMNI_OK;
-    case OMNI_EXPERT_ALGO_SPLIT: return (split_lanes_per_row(H, es) != 0 && k <= 2 * kWave) ? OMNI_OK : OMNI_ERR_UNSUPPORTED;
+    case OMNI_EXPERT_ALGO_AUTO:
+      if ((int64_t)H * es <= 8192) return OMNI_OK;
+      [[fallthrough]];                                           // wide rows: AUTO is the split algorithm
+    case OMNI_EXPERT_ALGO_SPLIT: {
+      int lpr = 0;
+      return (split_col_blocks(H, es, &lpr) != 0 && k <= 2 * kWave) ? OMNI_OK : OMNI_ERR_UNSUPPORTED;
+    }
+    case OMNI_EXPERT_ALGO_GATHER: case OMNI_EXPERT_ALGO_SEGMENT: return (int64_t)H * es <= 8192 ? OMNI_OK : OMNI_ERR_UNSUPPORTED;
     case OMNI_EXPERT_ALGO_DENSE: return (k == 0 || T == 0 || dense_covers(T, H, N, k, dtype)) ? OMNI_OK : OMNI_ERR_UNSUPPORTED;
     default: return OMNI_ERR_UNSUPPORTED;
   }
@@ -556,8 +582,11 @@ extern "C" OMNI_API size_t omni_expert_workspace_bytes(int64_t num_tokens, int32
                                                        int32_t num_experts_per_token, int32_t dtype, int32_t algo) {
   if (num_tokens < 0 || num_experts <= 0 || num_experts_per_token < 0) return 0;
   algo = omni::resolve_algo(algo, num_tokens, hidden_size, num_experts, num_experts_per_token, dtype);
-  if (algo == OMNI_EXPERT_ALGO_SPLIT)
-    return omni::align256((size_t)omni::kSlices * (size_t)num_tokens * (size_t)num_experts_per_token * 4);
+  if (algo == OMNI_EXPERT_ALGO_SPLIT) {
+    int lpr = 0;
+    const int col_blocks = omni::split_col_blocks(hidden_size, dtype == OMNI_F32 ? 4 : 2, &lpr);
+    return omni::align256((size_t)omni::kSlices * (size_t)(col_blocks ? col_blocks : 1) * (size_t)num_tokens * (size_t)num_experts_per_token * 4);
+  }
   if (algo == OMNI_EXPERT_ALGO_DENSE)
     return omni::dense_covers(num_tokens, hidden_size, num_experts, num_experts_per_token, dtype) ? omni::dense_workspace_bytes(num_tokens, hidden_size, num_experts) : 0;
   if (algo != OMNI_EXPERT_ALGO_SEGMENT) return 0;   // the gather algorithm keeps everything in registers

@@ -70,7 +70,7 @@ extern "C" OMNI_API int32_t omni_moe_fwd_algo(const void* x, const void* gate_we
     const int64_t esz = (int64_t)elem_bytes(dtype), r = num_expert_sqrt, k = num_experts_per_token;
     if ((hidden_size * esz) % 16 != 0 || (intermediate_size * esz) % 16 != 0) return OMNI_ERR_SHAPE;   // rows are fetched 16 bytes at a time
     if (k < 0 || k > r * r || k > 128 || k % 2 != 0) return OMNI_ERR_TOPK;
-    if (r > 1024 || hidden_size * esz > 8192) return OMNI_ERR_UNSUPPORTED;
+    if (r > 1024) return OMNI_ERR_UNSUPPORTED;
     if (r * r > num_experts) return OMNI_ERR_SHAPE;                                                   // ids reach r*r - 1
     if (int e = expert_algo_check(expert_algo, num_tokens, hidden_size, num_experts, num_experts_per_token, dtype)) return e;
   }

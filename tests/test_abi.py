@@ -78,7 +78,7 @@ def test_argument_errors_need_no_gpu():
     assert moe(64, 64, 16, 4, 3) == -4           # odd k
     assert moe(64, 64, 16, 4, 18) == -4          # k > r*r
     assert moe(64, 64, 15, 4, 2) == -2           # r*r experts do not fit the tables
-    assert moe(8192, 64, 16, 4, 2) == -5         # rows beyond 8 KiB
+    assert moe(8200, 64, 16, 4, 2) == -5         # 16 400-byte rows: no cut into column blocks of 8 power-of-two slices
     assert moe(64, 64, 16, 4, 2, dt=5) == -3
     assert lib.omni_mlp_fwd(p, p, p, p, None, p, 4, 64, 64, 0, None, None) == -6 # no workspace
     assert lib.omni_schedule_workspace_bytes(4, 2, 100) >= 200

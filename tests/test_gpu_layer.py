@@ -142,6 +142,7 @@ def test_router_fwd_select_is_exact_given_same_logprobs(device):
 
 LAYER_CASES = [
     # (T, H, I, N, k, seed)
+    (96, 8192, 256, 64, 4, 5),         # expert rows of 16 KiB: the split kernels in two column blocks
     (512, 256, 1024, 1024, 8, 0),      # benchmark config 1 shape, in bf16
     (4096, 1024, 4096, 4096, 16, 3),   # benchmark config 4 (README shape)
     (300, 128, 256, 1000, 8, 1),       # N not a square: r = floor(sqrt(N)) = 31 (omni_moe.py:38), odd, ids < 961
