@@ -230,7 +230,7 @@ __device__ __forceinline__ void count_batch(const SelectArgs& g) {
     for (int i = threadIdx.x; i < 2 * g.r; i += blockDim.x) {
       const int half = i >= g.r, key = i - half * g.r;
       g.stats_out[(2 * half) * g.r + key] = load_score(g.run_mean[half], key, g.stat_dt);
-      g.stats_out[(2 * half + 1) * g.r + key] = 1.0f / sqrtf(load_score(g.run_var[half], key, g.stat_dt) + g.eps);
+      g.stats_out[(2 * half + 1) * g.r + key] = __builtin_amdgcn_rsqf(load_score(g.run_var[half], key, g.stat_dt) + g.eps);
     }
   }
 }
@@ -249,9 +249,9 @@ __device__ __forceinline__ void normalise_half(float (&v)[R], const SelectArgs& 
       if (g.stats) {
         mean = g.stats[(2 * half) * r + key];
         rstd = g.stats[(2 * half + 1) * r + key];
-      } else {                                   // the same expressions as bn_finalize_kernel's
+      } else {                                   // per token and key: the hardware's reciprocal square root (1 ulp), as in stats_out
         mean = load_score(g.run_mean[half], key, g.stat_dt);
-        rstd = 1.0f / sqrtf(load_score(g.run_var[half], key, g.stat_dt) + g.eps);
+        rstd = __builtin_amdgcn_rsqf(load_score(g.run_var[half], key, g.stat_dt) + g.eps);
       }
       v[a] = round_score((v[a] - mean) * rstd, dt);
     }
@@ -421,6 +421,33 @@ __device__ __forceinline__ void ksizes(uint32_t (&k0)[R], uint32_t (&k1)[R], con
 template <int R> __device__ __forceinline__ void ksort(uint32_t (&k)[R], const int lane) { ksizes<R, 2>(k, k, lane, false); }
 template <int R> __device__ __forceinline__ void ksort2(uint32_t (&k0)[R], uint32_t (&k1)[R], const int lane) { ksizes<R, 2>(k0, k1, lane, true); }
 
+// The 64 largest keys of each list (64*R keys, item = reg*64 + lane), descending, into register 0 -- all that the
+// candidate stage reads when k' <= 64.  Every register is sorted across the lanes by itself (compile-time lane
+// distances, no LDS), then the registers are merged pairwise: for two descending runs A and B, max(A[i], B[63-i])
+// holds the 64 largest of both as a bitonic sequence, which six more compare-exchange steps put in order.  About a
+// third of the compare-exchanges of a full sort of 512 keys, and none of them through run-time lane distances.
+template <int R>
+__device__ __forceinline__ void ktop64_2(uint32_t (&k0)[R], uint32_t (&k1)[R], const int lane) {
+#pragma unroll
+  for (int a = 0; a < R; ++a) {
+    uint32_t x[1] = {k0[a]}, y[1] = {k1[a]};
+    ksizes<1, 2>(x, y, lane, true);
+    k0[a] = x[0];
+    k1[a] = y[0];
+  }
+#pragma unroll
+  for (int width = R; width > 1; width /= 2) {
+#pragma unroll
+    for (int a = 0; a < width / 2; ++a) {
+      uint32_t x[1] = {max(k0[a], (uint32_t)__shfl((int)k0[a + width / 2], 63 - lane, kWave))};
+      uint32_t y[1] = {max(k1[a], (uint32_t)__shfl((int)k1[a + width / 2], 63 - lane, kWave))};
+      kstages_ct<1, kWave, kWave / 2>(x, y, lane, true);
+      k0[a] = x[0];
+      k1[a] = y[0];
+    }
+  }
+}
+
 template <int R>
 __device__ __forceinline__ uint32_t sorted_key(const uint32_t (&v)[R], int i) {
   uint32_t r0 = (uint32_t)__shfl((int)v[0], i & 63, kWave);
@@ -473,7 +500,8 @@ __global__ __launch_bounds__(kRouterWaves* kWave) void router_select_packed_kern
       kx[a] = key < r ? make_key(sx[a], key, dt) : 0u;          // 0 sorts behind every real key
       ky[a] = key < r ? make_key(sy[a], key, dt) : 0u;
     }
-    ksort2<R>(kx, ky, lane);
+    if (R > kUnrollMaxR && kp <= kWave) ktop64_2<R>(kx, ky, lane);    // uniform: kp comes with the arguments
+    else ksort2<R>(kx, ky, lane);
 
     uint32_t ck[C];
 #pragma unroll
