@@ -267,7 +267,54 @@ __device__ __forceinline__ void normalise_half(float (&v)[R], const SelectArgs& 
     if (a * kWave + lane < r) v[a] = round_score(v[a] - m - lse, dt);
 }
 
-// R = half keys per lane (r <= 64*R); C = candidate cells per lane.
+// This lane's candidate cells: cell index ci = c*64+lane enumerates rows a = 0..kp-1 with
+// min(kp, k/(a+1)) cells each.  Payload (a<<8)|b orders like position a*kp+b.  The row counts
+// come with the arguments: the lanes fetch them all at once (row a in lane a%64) and the uniform
+// loop hands them round by readlane, so it waits for memory once, not once per row.
+template <int R, int C>
+__device__ __forceinline__ void candidate_cells(int (&cell)[C], const SelectArgs& g, const int kp, const int lane) {
+#pragma unroll
+  for (int c = 0; c < C; ++c) cell[c] = -1;
+  // Measured per shape: with 4 or 8 keys and fewer than 8 cells per lane the plain loop, one load per row, is the faster
+  // one by 3-6 % of the kernel (32768 tokens, 256-512 keys per half, k = 32); everywhere else the lanes' loop is, by 1-6 %.
+  if constexpr (R > 2 && C < 8) {
+    for (int a = 0, start = 0; a < kp; ++a) {
+      const int cnt = g.row_cells[a];
+#pragma unroll
+      for (int c = 0; c < C; ++c) {
+        const int b = c * kWave + lane - start;
+        cell[c] = (unsigned)b < (unsigned)cnt ? (a << 8) | b : cell[c];
+      }
+      start += cnt;
+    }
+    return;
+  }
+  const int cnt_lo = lane < kp ? g.row_cells[lane] : 0;
+  const int cnt_hi = lane + kWave < kp ? g.row_cells[lane + kWave] : 0;
+  int start = 0;
+  for (int a = 0; a < min(kp, kWave); ++a) {
+    const int cnt = __builtin_amdgcn_readlane(cnt_lo, a);
+#pragma unroll
+    for (int c = 0; c < C; ++c) {
+      const int b = c * kWave + lane - start;
+      cell[c] = (unsigned)b < (unsigned)cnt ? (a << 8) | b : cell[c];
+    }
+    start += cnt;
+  }
+  for (int a = kWave; a < kp; ++a) {
+    const int cnt = __builtin_amdgcn_readlane(cnt_hi, a - kWave);
+#pragma unroll
+    for (int c = 0; c < C; ++c) {
+      const int b = c * kWave + lane - start;
+      cell[c] = (unsigned)b < (unsigned)cnt ? (a << 8) | b : cell[c];
+    }
+    start += cnt;
+  }
+}
+
+// R = half keys per lane (r <= 64*R); C = candidate cells per lane.  With few keys per lane a wave requests
+// the raw scores of its first token before anything else and those of its next token as soon as the current
+// token's are consumed.
 template <int R, int C>
 __global__ __launch_bounds__(kRouterWaves* kWave) void router_select_kernel(const SelectArgs g) {
   count_batch(g);
@@ -276,20 +323,20 @@ __global__ __launch_bounds__(kRouterWaves* kWave) void router_select_kernel(cons
   const int num_waves = gridDim.x * kRouterWaves;
   const int r = g.r, k = g.k, kp = g.kp, dt = g.dt;
 
-  // This lane's candidate cells: cell index ci = c*64+lane enumerates rows a = 0..kp-1
-  // with min(kp, k/(a+1)) cells each.  Payload (a<<8)|b orders like position a*kp+b.
-  int cell[C];
+  float rx[R], ry[R];                             // raw scores of the token about to be selected
+  auto load_raw = [&](int t) __attribute__((always_inline)) {
 #pragma unroll
-  for (int c = 0; c < C; ++c) cell[c] = -1;
-  for (int a = 0, start = 0; a < kp; ++a) {       // uniform loop, counts come with the arguments
-    const int cnt = g.row_cells[a];
-#pragma unroll
-    for (int c = 0; c < C; ++c) {
-      const int b = c * kWave + lane - start;
-      cell[c] = (unsigned)b < (unsigned)cnt ? (a << 8) | b : cell[c];
+    for (int a = 0; a < R; ++a) {
+      const int key = a * kWave + lane;
+      const bool ok = key < r;
+      rx[a] = ok ? load_score(g.lx, int64_t(t) * g.row_stride + key, dt) : kNegInf;
+      ry[a] = ok ? load_score(g.ly, int64_t(t) * g.row_stride + key, dt) : kNegInf;
     }
-    start += cnt;
-  }
+  };
+  constexpr bool kPrefetch = R <= 2;              // beyond that the extra live registers cost a wave per SIMD
+  if (kPrefetch && wave < g.num_tokens) load_raw(wave);
+  int cell[C];
+  candidate_cells<R, C>(cell, g, kp, lane);
 
   for (int t = wave; t < g.num_tokens; t += num_waves) {
     float sx[R], sy[R];
@@ -298,10 +345,11 @@ __global__ __launch_bounds__(kRouterWaves* kWave) void router_select_kernel(cons
     for (int a = 0; a < R; ++a) {
       const int key = a * kWave + lane;
       const bool ok = key < r;
-      sx[a] = ok ? load_score(g.lx, int64_t(t) * g.row_stride + key, dt) : kNegInf;
-      sy[a] = ok ? load_score(g.ly, int64_t(t) * g.row_stride + key, dt) : kNegInf;
+      sx[a] = kPrefetch ? rx[a] : ok ? load_score(g.lx, int64_t(t) * g.row_stride + key, dt) : kNegInf;
+      sy[a] = kPrefetch ? ry[a] : ok ? load_score(g.ly, int64_t(t) * g.row_stride + key, dt) : kNegInf;
       px[a] = py[a] = key;
     }
+    if (kPrefetch && t + num_waves < g.num_tokens) load_raw(t + num_waves);
     if (g.stats || g.run_mean[0]) {
       normalise_half<R>(sx, g, 0, r, lane, dt);
       normalise_half<R>(sy, g, 1, r, lane, dt);
@@ -467,18 +515,20 @@ __global__ __launch_bounds__(kRouterWaves* kWave) void router_select_packed_kern
   const int num_waves = gridDim.x * kRouterWaves;
   const int r = g.r, k = g.k, kp = g.kp, dt = g.dt;
 
-  int cell[C];                                  // as in router_select_kernel
+  float rx[R], ry[R];                             // as in router_select_kernel
+  auto load_raw = [&](int t) __attribute__((always_inline)) {
 #pragma unroll
-  for (int c = 0; c < C; ++c) cell[c] = -1;
-  for (int a = 0, start = 0; a < kp; ++a) {       // uniform loop, counts come with the arguments
-    const int cnt = g.row_cells[a];
-#pragma unroll
-    for (int c = 0; c < C; ++c) {
-      const int b = c * kWave + lane - start;
-      cell[c] = (unsigned)b < (unsigned)cnt ? (a << 8) | b : cell[c];
+    for (int a = 0; a < R; ++a) {
+      const int key = a * kWave + lane;
+      const bool ok = key < r;
+      rx[a] = ok ? load_score(g.lx, int64_t(t) * g.row_stride + key, dt) : kNegInf;
+      ry[a] = ok ? load_score(g.ly, int64_t(t) * g.row_stride + key, dt) : kNegInf;
     }
-    start += cnt;
-  }
+  };
+  constexpr bool kPrefetch = R <= 2;              // beyond that the extra live registers cost a wave per SIMD
+  if (kPrefetch && wave < g.num_tokens) load_raw(wave);
+  int cell[C];
+  candidate_cells<R, C>(cell, g, kp, lane);
 
   for (int t = wave; t < g.num_tokens; t += num_waves) {
     float sx[R], sy[R];
@@ -486,9 +536,10 @@ __global__ __launch_bounds__(kRouterWaves* kWave) void router_select_packed_kern
     for (int a = 0; a < R; ++a) {
       const int key = a * kWave + lane;
       const bool ok = key < r;
-      sx[a] = ok ? load_score(g.lx, int64_t(t) * g.row_stride + key, dt) : kNegInf;
-      sy[a] = ok ? load_score(g.ly, int64_t(t) * g.row_stride + key, dt) : kNegInf;
+      sx[a] = kPrefetch ? rx[a] : ok ? load_score(g.lx, int64_t(t) * g.row_stride + key, dt) : kNegInf;
+      sy[a] = kPrefetch ? ry[a] : ok ? load_score(g.ly, int64_t(t) * g.row_stride + key, dt) : kNegInf;
     }
+    if (kPrefetch && t + num_waves < g.num_tokens) load_raw(t + num_waves);
     if (g.stats || g.run_mean[0]) {
       normalise_half<R>(sx, g, 0, r, lane, dt);
       normalise_half<R>(sy, g, 1, r, lane, dt);
@@ -587,13 +638,7 @@ struct BnFinalArgs {
   float momentum, eps;               // momentum < 0: cumulative moving average, factor 1 / (batches tracked so far + 1)
 };
 
-__device__ __forceinline__ double wave_sum_f64(double v) {
-#pragma unroll
-  for (int m = kWave / 2; m >= 1; m >>= 1) v += __shfl_xor(v, m, kWave);
-  return v;
-}
-
-// One wave per column: merges the strip partials exactly (mean = sum n_s mean_s / n,
+// One wave per column: merges the strip partials (mean = sum n_s mean_s / n,
 // M2 = sum M2_s + n_s (mean_s - mean)^2, in double), writes mean and 1/sqrt(var+eps), and in
 // training moves the running buffers (unbiased variance) as nn.BatchNorm1d does.  In eval
 // the running buffers provide mean and variance.
@@ -607,16 +652,23 @@ __global__ __launch_bounds__(256) void bn_finalize_kernel(const BnFinalArgs g) {
   const int half = col >= g.r, key = col - half * g.r;
   float mean, var;
   if (g.training) {
-    double wsum = 0.;
-    for (int s = lane; s < g.strips; s += kWave)
-      wsum += (double)min(kBnRows, g.num_rows - s * kBnRows) * (double)g.part_mean[int64_t(s) * 2 * g.r + col];
-    const double n = (double)g.num_rows, mu = wave_sum_f64(wsum) / n;
-    double q = 0.;
+    // one pass over the strips, both sums in double: M2 = sum (M2_s + n_s mean_s^2) - n mu^2 (double carries 29 bits more than
+    // the fp32 result keeps, so the difference stays exact to fp32 while mean^2 / variance < 2^29)
+    double wsum = 0., q = 0.;
     for (int s = lane; s < g.strips; s += kWave) {
-      const double d = (double)g.part_mean[int64_t(s) * 2 * g.r + col] - mu;
-      q += (double)g.part_m2[int64_t(s) * 2 * g.r + col] + (double)min(kBnRows, g.num_rows - s * kBnRows) * d * d;
+      const double ns = (double)min(kBnRows, g.num_rows - s * kBnRows), ms = (double)g.part_mean[int64_t(s) * 2 * g.r + col];
+      wsum += ns * ms;
+      q += (double)g.part_m2[int64_t(s) * 2 * g.r + col] + ns * ms * ms;
     }
-    const double m2 = wave_sum_f64(q);
+    double sum2[2] = {wsum, q};
+#pragma unroll
+    for (int m = kWave / 2; m >= 1; m >>= 1) {
+      const double o0 = __shfl_xor(sum2[0], m, kWave), o1 = __shfl_xor(sum2[1], m, kWave);
+      sum2[0] += o0;
+      sum2[1] += o1;
+    }
+    const double n = (double)g.num_rows, mu = sum2[0] / n;
+    const double m2 = fmax(sum2[1] - n * mu * mu, 0.);
     mean = (float)mu;
     var = (float)(m2 / n);                                   // biased: normalises the batch
     if (lane == 0) {
