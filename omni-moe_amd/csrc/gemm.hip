@@ -10,6 +10,9 @@
 // on 8 waves (2 x 4, two per SIMD) of 128 x 64 instead.  16-bit operands with K % 64 == 0
 // take `gemm_nt_dma_kernel` (global -> LDS directly, ring of stages, swizzled rows); anything
 // else takes `gemm_nt_kernel` (global -> registers -> one of two LDS stages with padded rows).
+// Two more forms of the direct-to-LDS kernel: `gemm_stream_kernel` (the 256 x 256 tile, one block per CU
+// walking its output tiles) and `gemm_ksplit_kernel` (fewer 64 x 64 tiles than CUs: a block's waves share
+// out the K tiles).
 // The weight fragment is the MFMA's first operand, so an accumulator lane holds 4 consecutive
 // output columns of one row; two lanes pair up to store 8 columns (16 bytes) each.
 #include "common.h"
@@ -789,6 +792,127 @@ __global__ __launch_bounds__(512, 1) void gemm_stream_kernel(const GemmArgs g) {
   }
 }
 
+// ---- few output tiles, long K: the K tiles of one 64 x 64 output tile dealt out over the block's four waves ----------
+// A product like the router projection at a few thousand tokens (4096 x 128 x 1024) has too few output tiles to fill the
+// GPU and its time is the latency of one block's K loop: with the ring kernel above, 16 rounds of wait - barrier - four
+// MFMAs.  Here every wave multiplies the whole 64 x 64 tile (2 x 2 MFMA tiles) over ITS K tiles (kt = wave, wave + 4,
+// ...) through a two-stage LDS ring of its own, so the K loop is a quarter as long, has four independent accumulators
+// to keep the matrix pipeline fed, and meets no block barrier: a wave waits only for its own loads.  The four partial
+// tiles then meet in LDS (summed in wave order, so the result does not depend on timing), and wave w finishes MFMA tile
+// (w % 2, w / 2) with the common epilogue.  Needs K % 64 == 0; worth it while there are fewer tiles than CUs.
+template <int DT, int EPI>
+__global__ __launch_bounds__(kGemmThreads, 1) void gemm_ksplit_kernel(const GemmArgs g) {
+  constexpr int kRow = 128, kTile = 64 * kRow;          // one operand's 64 rows of a K tile
+  constexpr int kStage = 2 * kTile, kRing = 2 * kStage; // per wave: two stages of [activations | weights]
+  extern __shared__ __align__(16) uint8_t lds[];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int tile_m = blockIdx.x % g.tiles_m, tile_n = blockIdx.x / g.tiles_m;
+  const int m0 = tile_m * 64, n0 = tile_n * 64;
+  uint8_t* ring = lds + wave * kRing;
+
+  // load instruction p (0..7) fills rows 8p + lane/8 of an operand tile; the lane fetches the logical chunk that belongs at
+  // its (swizzled) position
+  const uint8_t* a_src[8];
+  const uint8_t* b_src[8];
+#pragma unroll
+  for (int p = 0; p < 8; ++p) {
+    const int rl = p * 8 + (lane >> 3);
+    const int c = swizzle<64>(rl, lane & 7);
+    int row = m0 + rl;
+    row = row < g.M ? row : g.M - 1;                    // clamp: tail rows and columns are never stored
+    a_src[p] = g.a + ((int64_t)row * g.K + c * 8) * 2;
+    int col = n0 + rl;
+    col = col < g.N ? col : g.N - 1;
+    const uint8_t* base = g.b0;
+    if constexpr (EPI == kEpiPlain || EPI == kEpiStats) {
+      if (g.b1 && col >= g.N / 2) { base = g.b1; col -= g.N / 2; }
+    }
+    b_src[p] = base + ((int64_t)col * g.K + c * 8) * 2;
+  }
+  auto issue_tile = [&](int kt, int stage) __attribute__((always_inline)) {
+    uint8_t* st = ring + stage * kStage;
+    const int koff = kt * kRow;
+#pragma unroll
+    for (int p = 0; p < 8; ++p)
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(a_src[p] + koff),
+                                       (__attribute__((address_space(3))) void*)(st + p * 1024), 16, 0, 0);
+#pragma unroll
+    for (int p = 0; p < 8; ++p)
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(b_src[p] + koff),
+                                       (__attribute__((address_space(3))) void*)(st + kTile + p * 1024), 16, 0, 0);
+  };
+
+  // fragment reads: lane reads row lane%32 (+32 i), logical chunk 2*slab + lane/32
+  const int rl = lane & 31;
+  int off_slab[4];
+#pragma unroll
+  for (int sl = 0; sl < 4; ++sl) off_slab[sl] = rl * kRow + swizzle<64>(rl, 2 * sl + (lane >> 5)) * 16;
+
+  f32x16_t acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int q = 0; q < 16; ++q) acc[i][j][q] = 0.f;
+
+  const int num_kt = g.K / 64;
+  const int mine = (num_kt - wave + 3) / 4;             // K tiles wave, wave + 4, ...
+  if (mine > 0) issue_tile(wave, 0);
+  if (mine > 1) issue_tile(wave + 4, 1);
+  for (int t = 0; t < mine; ++t) {
+    if (t + 1 < mine) wait_vmcnt<16>(); else wait_vmcnt<0>();     // this tile has landed; the next one may be in flight
+    const uint8_t* st = ring + (t & 1) * kStage;
+    u32x4_t af[2][2], bf[2][2];
+    auto read_slab = [&](int sl) __attribute__((always_inline)) {
+#pragma unroll
+      for (int i = 0; i < 2; ++i) af[sl & 1][i] = *(const u32x4_t*)(st + off_slab[sl] + i * 32 * kRow);
+#pragma unroll
+      for (int j = 0; j < 2; ++j) bf[sl & 1][j] = *(const u32x4_t*)(st + kTile + off_slab[sl] + j * 32 * kRow);
+    };
+    read_slab(0);
+#pragma unroll
+    for (int sl = 0; sl < 4; ++sl) {
+      if (sl + 1 < 4) read_slab(sl + 1);
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = mfma32<DT>(bf[sl & 1][j], af[sl & 1][i], acc[i][j]);
+    }
+    if (t + 2 < mine) {
+      wait_lds_reads();                                  // the stage is read out (by this wave, its only reader)
+      issue_tile(wave + 4 * (t + 2), t & 1);
+    }
+  }
+
+  // ---- the four partial tiles meet in LDS: [wave][MFMA tile][column group][lane] 16 bytes each
+  __syncthreads();                                       // every wave is done with its ring
+  f32x4_t* xch = (f32x4_t*)lds;
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4)
+        xch[((wave * 4 + (j * 2 + i)) * 4 + q4) * 64 + lane] =
+            f32x4_t{acc[i][j][q4 * 4], acc[i][j][q4 * 4 + 1], acc[i][j][q4 * 4 + 2], acc[i][j][q4 * 4 + 3]};
+  __syncthreads();
+  f32x16_t sum[1][1];
+#pragma unroll
+  for (int q4 = 0; q4 < 4; ++q4) {
+    f32x4_t v = xch[((0 * 4 + wave) * 4 + q4) * 64 + lane];
+#pragma unroll
+    for (int w = 1; w < 4; ++w) {
+      const f32x4_t o = xch[((w * 4 + wave) * 4 + q4) * 64 + lane];
+      v[0] += o[0]; v[1] += o[1]; v[2] += o[2]; v[3] += o[3];
+    }
+    sum[0][0][q4 * 4] = v[0]; sum[0][0][q4 * 4 + 1] = v[1]; sum[0][0][q4 * 4 + 2] = v[2]; sum[0][0][q4 * 4 + 3] = v[3];
+  }
+  gemm_epilogue<DT, 1, 1, EPI>(g, sum, m0, n0, wave & 1, wave >> 1, lane);
+}
+
 // One list entry per kernel instantiation that launch_gemm can start (the static members come into being
 // at library load for every instantiation the dispatch below names).
 template <int DT, int TM, int TN, int EPI, int BK, int NS, int NW = 4>
@@ -798,6 +922,10 @@ struct DmaKernelLds {
 template <int DT, int EPI>
 struct StreamKernelLds {
   static inline LdsKernel entry{(const void*)gemm_stream_kernel<DT, EPI>, 2 * 512 * 128};
+};
+template <int DT, int EPI>
+struct KsplitKernelLds {
+  static inline LdsKernel entry{(const void*)gemm_ksplit_kernel<DT, EPI>, 4 * 2 * 2 * 64 * 128};
 };
 template <int DT, int TM, int TN, int EPI>
 struct StagedKernelLds {
@@ -838,6 +966,14 @@ static hipError_t launch_gemm(GemmArgs g, hipStream_t s) {
       if (covers) {
         if (hipError_t e = StreamKernelLds<DT, EPI>::entry.ensure(); e != hipSuccess) return e;
         hipLaunchKernelGGL((gemm_stream_kernel<DT, EPI>), dim3(256), dim3(512), 2 * 512 * 128, s, g);
+        return hipGetLastError();
+      }
+    }
+    if constexpr (TM == 1 && TN == 1 && EPI != kEpiSwiglu && EPI != kEpiGate) {
+      // fewer 64 x 64 tiles than CUs and at least two K tiles per wave: the K tiles dealt out over the waves
+      if (blocks <= 256 && g.K >= 512) {
+        if (hipError_t e = KsplitKernelLds<DT, EPI>::entry.ensure(); e != hipSuccess) return e;
+        hipLaunchKernelGGL((gemm_ksplit_kernel<DT, EPI>), dim3(blocks), dim3(kGemmThreads), 4 * 2 * 2 * 64 * 128, s, g);
         return hipGetLastError();
       }
     }

@@ -67,7 +67,7 @@ def test_mlp_fp32_matches_oracle(case, device):
 
 
 # the last two make the projection GEMM pick its 128 x 128 and 256 x 256 tiles (statistics epilogue included)
-ROUTER_FWD_CASES = [(4096, 1024, 64, 16), (1024, 256, 32, 8), (2048, 2048, 512, 32), (300, 520, 36, 10),
+ROUTER_FWD_CASES = [(4096, 1024, 64, 16), (1024, 256, 32, 8), (2048, 2048, 512, 32), (300, 520, 36, 10), (300, 576, 36, 10),
                     (4096, 256, 512, 32), (16384, 256, 512, 32)]
 
 
@@ -405,7 +405,9 @@ def test_add_inplace(device):
 # included; then a big-tile case, N % 8 == 4 (rows written 8 bytes per lane instead of 16), a ragged last column tile
 LINEAR_CASES = [(3300, 1024, 512), (3300, 1024, 640), (3300, 1024, 576), (4096, 1024, 4096), (2049, 1536, 1024),
                 (4096, 4096, 256), (300, 100, 264), (333, 1000, 256), (70, 4, 8),
-                (300, 62, 128), (129, 1001, 64), (70, 6, 16), (5, 1, 8)]       # N % 4 != 0: element-wise stores
+                (300, 62, 128), (129, 1001, 64), (70, 6, 16), (5, 1, 8),       # N % 4 != 0: element-wise stores
+                # few 64 x 64 tiles and K >= 512: the K tiles of a block dealt out over its waves (even and ragged shares, tails)
+                (4096, 128, 1024), (1000, 104, 512), (130, 72, 640), (64, 64, 4096), (200, 6, 576), (33, 250, 832)]
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
