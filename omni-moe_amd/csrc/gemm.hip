@@ -11,8 +11,8 @@
 // take `gemm_nt_dma_kernel` (global -> LDS directly, ring of stages, swizzled rows); anything
 // else takes `gemm_nt_kernel` (global -> registers -> one of two LDS stages with padded rows).
 // Two more forms of the direct-to-LDS kernel: `gemm_stream_kernel` (the 256 x 256 tile, one block per CU
-// walking its output tiles) and `gemm_ksplit_kernel` (fewer 64 x 64 tiles than CUs: a block's waves share
-// out the K tiles).
+// walking its output tiles, on 16x16x32 MFMAs) and `gemm_ksplit_kernel` (fewer 64 x 64 tiles than CUs: a
+// block's waves share out the K tiles).
 // The weight fragment is the MFMA's first operand, so an accumulator lane holds 4 consecutive
 // output columns of one row; two lanes pair up to store 8 columns (16 bytes) each.
 #include "common.h"
@@ -634,11 +634,19 @@ __global__ __launch_bounds__(NW * 64, 1) void gemm_nt_dma_kernel(const GemmArgs 
 // One block per CU walks its share of the output tiles (tile index blockIdx, blockIdx + gridDim, ...).  The K tiles of
 // consecutive output tiles form ONE stream through the two LDS stages: while a block multiplies the last K tiles of an
 // output tile, the first K tiles of its next one are already on their way, so only a block's first output tile waits for
-// memory before its first matrix instruction (gate/up projection at 4096 x 4096 x 1024, two tiles per block: 62.9 us
-// against 65.3 us; 32768 x 16384 x 2048: 1.82 against 1.87 ms).  Ring loads are buffer loads (scalar base and tile
-// offsets, one 32-bit lane offset per operand).  The grid keeps every CU until the kernel ends, so a kernel on another
-// stream finds no room beside it: the callers use this form where nothing is meant to run concurrently.
+// memory before its first matrix instruction.  Ring loads are buffer loads (scalar base and tile offsets, one 32-bit
+// lane offset per operand).  The grid keeps every CU until the kernel ends, so a kernel on another stream finds no room
+// beside it: the callers use this form where nothing is meant to run concurrently.
 // Needs full tiles (M % 256 == 0, N a multiple of the tile's columns), K % 64 == 0, whole rounds of 256 tiles.
+//
+// The wave's 128 x 64 tile is 8 x 4 MFMA tiles of 16 x 16 and K advances 32 per instruction.  Under sustained load the
+// board clocks by power, and on the same operand bits the 16 x 16 x 32 instruction sustains about 15 % more than
+// 32 x 32 x 16 (register-only probes, two waves per SIMD: 2.07 against 1.80 PFLOP/s; this kernel against the same
+// kernel on 32 x 32 x 16: 8192 x 8192 x 2048 207 against 222 us, 32768 x 2 x 8192 x 2048 with SwiGLU 1.66 against
+// 1.76 ms, 4096 x 2 x 4096 x 1024 level).  A lane of accumulator tile (i, j) holds row m = 16 i + lane%16 and the four
+// columns n = 16 j + 4 (lane/16) + 0..3.  The activation fragments are a single set that is refilled row by row (the
+// fragment of row tile i for the next K step is read as soon as row i's four instructions have issued); the weight
+// fragments alternate between two sets.
 __device__ __forceinline__ void tile_coords_of(const GemmArgs& g, int b, int& tile_m, int& tile_n) {
   if (g.patch_m > 0) {
     const int per_patch = g.patch_m * g.patch_n;
@@ -653,9 +661,66 @@ __device__ __forceinline__ void tile_coords_of(const GemmArgs& g, int b, int& ti
   }
 }
 
+template <int DT>
+__device__ __forceinline__ f32x4_t mfma16(const u32x4_t a, const u32x4_t b, f32x4_t c) {
+  if constexpr (DT == kBF16) return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+  else return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+}
+
+// Epilogue of the streaming kernel (full tiles, 16-byte stores).  Lanes l and l ^ 16 hold columns 4g..4g+3 and 4g+4..4g+7 of
+// two neighbouring column tiles: one v_permlane16_swap per word leaves every lane with 8 consecutive columns of one
+// of the two tiles, so each store instruction writes 64 consecutive bytes of 16 rows.
+template <int DT, int EPI>
+__device__ __forceinline__ void stream_epilogue(const GemmArgs& g, f32x4_t (&acc)[8][4], const int m0, const int n0, const int wm,
+                                                  const int wn, const int lane) {
+  constexpr int TNO = (EPI == kEpiSwiglu) ? 2 : 4;
+  const int g4 = lane >> 4;
+  const int nb = n0 + wn * (TNO * 16);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int m = m0 + wm * 128 + i * 16 + (lane & 15);
+#pragma unroll
+    for (int j = 0; j < TNO; j += 2) {
+      uint32_t w[2][2];
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        float v[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          if constexpr (EPI == kEpiSwiglu) {
+            // gate and up are materialised in the storage dtype, silu(gate)*up is formed in fp32 and rounded once (omni_mlp.py:53-61)
+            const float gt = Elem<DT>::round(acc[i][j + t][q]), up = Elem<DT>::round(acc[i][j + t + TNO][q]);
+            v[q] = silu_fast(gt) * up;
+          } else {
+            v[q] = acc[i][j + t][q];
+          }
+        }
+        if constexpr (EPI == kEpiResidual) {
+          const u32x2_t r = *(const u32x2_t*)(g.res + ((int64_t)m * g.N + nb + (j + t) * 16 + g4 * 4) * 2);
+          const uint32_t r0 = r[0], r1 = r[1];
+          if constexpr (DT == kBF16) {
+            v[0] = Elem<DT>::round(v[0]) + bf16_lo(r0); v[1] = Elem<DT>::round(v[1]) + bf16_hi(r0);
+            v[2] = Elem<DT>::round(v[2]) + bf16_lo(r1); v[3] = Elem<DT>::round(v[3]) + bf16_hi(r1);
+          } else {
+            v[0] = Elem<DT>::round(v[0]) + f16_bits_to_f32(r0 & 0xffff); v[1] = Elem<DT>::round(v[1]) + f16_bits_to_f32(r0 >> 16);
+            v[2] = Elem<DT>::round(v[2]) + f16_bits_to_f32(r1 & 0xffff); v[3] = Elem<DT>::round(v[3]) + f16_bits_to_f32(r1 >> 16);
+          }
+        }
+        w[t][0] = pack2<DT>(v[0], v[1]);
+        w[t][1] = pack2<DT>(v[2], v[3]);
+      }
+      // odd 16-lane rows of tile j's words change places with even rows of tile j+1's
+      const auto s0 = __builtin_amdgcn_permlane16_swap(w[0][0], w[1][0], false, false);
+      const auto s1 = __builtin_amdgcn_permlane16_swap(w[0][1], w[1][1], false, false);
+      const int n = nb + (j + (g4 & 1)) * 16 + (g4 & 2) * 4;
+      *(u32x4_t*)(g.c + ((int64_t)m * g.N + n) * 2) = u32x4_t{s0[0], s1[0], s0[1], s1[1]};
+    }
+  }
+}
+
 template <int DT, int EPI>
 __global__ __launch_bounds__(512, 1) void gemm_stream_kernel(const GemmArgs g) {
-  constexpr int TM = 4, TN = 2;                      // 8 waves as 2 x 4, each 128 x 64
+  constexpr int TM = 8, TN = 4;                      // MFMA tiles of 16 x 16 per wave: 128 x 64
   constexpr int BM = 256, BR = 256;
   constexpr int BN = (EPI == kEpiSwiglu) ? 128 : 256;
   constexpr int kRow = 128, kStage = (BM + BR) * kRow;
@@ -709,65 +774,81 @@ __global__ __launch_bounds__(512, 1) void gemm_stream_kernel(const GemmArgs g) {
     }
   };
 
-  // fragment reads: lane reads row lane%32, logical chunk 2*slab + lane/32, into buffer slab&1
-  const int rl = lane & 31;
-  int off_slab[4];
+  // fragment reads: lane reads row lane%16 of a 16-row tile, logical chunk 4*kstep + lane/16 (8 K values of the step's 32)
+  const int r16 = lane & 15;
+  int off_ks[2];
 #pragma unroll
-  for (int sl = 0; sl < 4; ++sl) off_slab[sl] = rl * kRow + swizzle<64>(rl, 2 * sl + (lane >> 5)) * 16;
-  const int a_frag = (wm * TM * 32) * kRow, b_frag = BM * kRow + (wn * TN * 32) * kRow;
-  u32x4_t af[2][TM], bf[2][TN];
-  auto read_one = [&](int stage, int slab, int f) __attribute__((always_inline)) {
-    const uint8_t* st = lds + stage * kStage + off_slab[slab];
-    if (f < TM) af[slab & 1][f] = *(const u32x4_t*)(st + a_frag + f * 32 * kRow);
-    else bf[slab & 1][f - TM] = *(const u32x4_t*)(st + b_frag + (f - TM) * 32 * kRow);
+  for (int ks = 0; ks < 2; ++ks) off_ks[ks] = r16 * kRow + ((4 * ks + (lane >> 4)) ^ (r16 >> 1)) * 16;
+  const int a_frag = (wm * 128) * kRow, b_frag = BM * kRow + (wn * 64) * kRow;
+  u32x4_t af[TM], bf[2][TN];
+  auto read_a = [&](int stage, int ks, int i) __attribute__((always_inline)) {
+    af[i] = *(const u32x4_t*)(lds + stage * kStage + a_frag + i * 16 * kRow + off_ks[ks]);
+  };
+  auto read_b = [&](int stage, int ks, int j) __attribute__((always_inline)) {
+    bf[ks][j] = *(const u32x4_t*)(lds + stage * kStage + b_frag + j * 16 * kRow + off_ks[ks]);
   };
 
-  f32x16_t acc[TM][TN];
+  f32x4_t acc[TM][TN];
   auto clear_acc = [&]() __attribute__((always_inline)) {
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
       for (int j = 0; j < TN; ++j)
 #pragma unroll
-        for (int q = 0; q < 16; ++q) acc[i][j][q] = 0.f;
+        for (int q = 0; q < 4; ++q) acc[i][j][q] = 0.f;
   };
   clear_acc();
 
-  // One slab: TM*TN matrix instructions, each followed by at most two memory instructions: the fragment reads of the
-  // following slab (stage read_stage) and, dma = 1 / 2, the activation / weight loads of the cursor's K tile.
-  auto slab = [&](auto sl_tag, auto next_tag, auto dma_tag, int read_stage) __attribute__((always_inline)) {
-    constexpr int sl = decltype(sl_tag)::value, next_slab = decltype(next_tag)::value, dma = decltype(dma_tag)::value;
-    const bool fv = dma == 1 ? f_tile < num_tiles : (dma == 2 && half_pending);
+  int c_stage = 0;                                     // stage of the K tile being multiplied
+  // One K step of 32: TM*TN matrix instructions in row order, at most one memory instruction behind each (slot_op).
+  // In the K tile's second step, whose following step reads the other stage, the wave waits after row 0 for its fragment
+  // reads and ring loads and meets the block.
+  constexpr int kSyncRow = 0;
+  // what follows matrix instruction (i, j): 0 nothing, 10+n weight fragment n, 20+n activation fragment n of the following
+  // step, 30+n ring load n of the cursor's K tile (0-3 activation rows, in the second step; 4-7 weight rows, in the first)
+  auto slot_op = [](bool second, int i, int j) constexpr -> int {
+    if (j == 0 && i >= 1 && i <= 4) return 10 + (i - 1);
+    if (j == 1 && i >= 1 && i <= 4) return second ? 30 + (i - 1) : 34 + (i - 1);
+    if (j == 2 && i == 1) return 20;
+    if (j == 3 && i >= 1) return 20 + i;
+    return 0;
+  };
+  auto kstep = [&](auto ks_tag, auto sync_tag) __attribute__((always_inline)) {
+    constexpr int ks = decltype(ks_tag)::value;
+    constexpr bool sync = decltype(sync_tag)::value;
+    constexpr int nks = ks ^ 1;
+    const int rs = sync ? c_stage ^ 1 : c_stage;      // stage the following step's fragments come from
+    const bool fa = f_tile < num_tiles;                // the cursor's K tile exists
 #pragma unroll
-    for (int ij = 0; ij < TM * TN; ++ij) {
-      const int i = ij / TN, j = ij % TN;
-      acc[i][j] = mfma32<DT>(bf[sl & 1][j], af[sl & 1][i], acc[i][j]);
-      __builtin_amdgcn_sched_barrier(0);
-      if (ij < TM + TN) read_one(read_stage, next_slab, ij);
-      if constexpr (dma != 0) {
-        if (ij >= TM + TN) {
-          const int q0 = (dma == 1 ? 0 : 4) + (ij - (TM + TN)) * 2;
-          if (fv) { issue_one(q0); issue_one(q0 + 1); }
+    for (int i = 0; i < TM; ++i) {
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        acc[i][j] = mfma16<DT>(bf[ks][j], af[i], acc[i][j]);
+        __builtin_amdgcn_sched_barrier(0);
+        const int op = slot_op(sync, i, j);
+        if (op >= 10 && op < 20) read_b(rs, nks, op - 10);
+        if (op >= 20 && op < 30) read_a(rs, nks, op - 20);
+        if (op >= 30 && op < 34) { if (fa) issue_one(op - 30); }
+        if (op >= 34) { if (half_pending) issue_one(op - 30); }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      if constexpr (sync) {
+        if (i == kSyncRow) {
+          wait_lds_reads();                            // this wave holds every fragment of the K tile
+          wait_vmcnt<0>();                             // the next K tile has landed
+          __builtin_amdgcn_s_barrier();                // ... for all waves; this K tile's stage is free
+          __builtin_amdgcn_sched_barrier(0);
         }
       }
-      __builtin_amdgcn_sched_barrier(0);
     }
   };
   using I0 = std::integral_constant<int, 0>; using I1 = std::integral_constant<int, 1>;
-  using I2 = std::integral_constant<int, 2>; using I3 = std::integral_constant<int, 3>;
-  int c_stage = 0;                                     // stage of the K tile being multiplied
-  // one K tile; on entry its slab-0 fragments are in registers
   auto k_tile = [&]() __attribute__((always_inline)) {
-    slab(I0{}, I1{}, I2{}, c_stage);                   // the weights of the K tile whose activations were requested one slab ago
+    kstep(I0{}, std::false_type{});                    // the weights of the K tile whose activations were requested one step ago
     if (half_pending) { cursor_advance(); half_pending = false; }
-    slab(I1{}, I2{}, I0{}, c_stage);
-    slab(I2{}, I3{}, I0{}, c_stage);
-    wait_lds_reads();                                  // this wave holds every fragment of the K tile
-    wait_vmcnt<0>();                                   // the next K tile has landed
-    __builtin_amdgcn_s_barrier();                      // ... for all waves; this K tile's stage is free
-    __builtin_amdgcn_sched_barrier(0);
-    half_pending = f_tile < num_tiles;
-    slab(I3{}, I0{}, I1{}, c_stage ^ 1);               // the activations of the K tile two ahead go into the freed stage
+    const bool fa = f_tile < num_tiles;
+    kstep(I1{}, std::true_type{});                     // the activations of the K tile two ahead go into the freed stage
+    half_pending = fa;
     c_stage ^= 1;
   };
 
@@ -781,13 +862,15 @@ __global__ __launch_bounds__(512, 1) void gemm_stream_kernel(const GemmArgs g) {
   wait_vmcnt<8>();                                     // the first K tile has landed
   __builtin_amdgcn_s_barrier();
 #pragma unroll
-  for (int f = 0; f < TM + TN; ++f) read_one(0, 0, f);
+  for (int i = 0; i < TM; ++i) read_a(0, 0, i);
+#pragma unroll
+  for (int j = 0; j < TN; ++j) read_b(0, 0, j);
 
   for (int tile = blockIdx.x; tile < num_tiles; tile += gridDim.x) {
     for (int kt = 0; kt < num_kt; ++kt) k_tile();
     int tm, tn;
     tile_coords_of(g, tile, tm, tn);
-    gemm_epilogue<DT, TM, TN, EPI>(g, acc, tm * BM, tn * BN, wm, wn, lane);
+    stream_epilogue<DT, EPI>(g, acc, tm * BM, tn * BN, wm, wn, lane);
     clear_acc();
   }
 }
