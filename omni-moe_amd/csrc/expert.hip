@@ -352,11 +352,14 @@ __global__ __launch_bounds__(kTokensPerBlock* kWave) void expert_split_dots_kern
 // Same ownership.  Lane `sub` of a group forms the coefficient of pair `sub` of a batch (sum of
 // the 8 slice partials in slice order, silu, gate); the group then walks the batch, every lane
 // fetching its 16 bytes of the down row and the pair's coefficient from the lane that holds it.
-template <int DT, int LPR>
+// WIDE: rows of several column blocks (col_block of col_blocks); otherwise both are compile-time constants, which keeps
+// the eight partial-sum loads of the common case one unrolled group that the compiler places behind the row requests.
+template <int DT, int LPR, bool WIDE>
 __global__ __launch_bounds__(kTokensPerBlock* kWave) void expert_split_accumulate_kernel(
     const uint8_t* __restrict__ down, const void* __restrict__ gates, const int32_t* __restrict__ ids,
     const float* __restrict__ partial, uint8_t* __restrict__ y, int num_tokens, int hidden, int top_k, uint32_t num_experts,
-    int col_block, int col_blocks) {
+    int col_block_arg, int col_blocks_arg) {
+  const int col_block = WIDE ? col_block_arg : 0, col_blocks = WIDE ? col_blocks_arg : 1;
   constexpr int E = Row16<DT>::kElems, GP = kWave / LPR;
   constexpr int LD = LPR < 8 ? LPR : 8;
   const int lane = lane_id(), sub = lane % LPR, grp = lane / LPR;
@@ -434,8 +437,13 @@ static hipError_t launch_split(const void* x, const void* up, const void* down, 
   for (int cb = 0; cb < col_blocks; ++cb)                            // all partial dot products first: a coefficient needs the whole row
     hipLaunchKernelGGL((expert_split_dots_kernel<DT, LPR>), dim3(blocks), dim3(kTokensPerBlock * kWave), 0, s, (const uint8_t*)x,
                        (const uint8_t*)up, ids, partial, (int)T, H, k, (uint32_t)N, cb);
+  if (col_blocks == 1) {
+    hipLaunchKernelGGL((expert_split_accumulate_kernel<DT, LPR, false>), dim3(blocks), dim3(kTokensPerBlock * kWave), 0, s,
+                       (const uint8_t*)down, gates, ids, partial, (uint8_t*)y, (int)T, H, k, (uint32_t)N, 0, 1);
+    return hipGetLastError();
+  }
   for (int cb = 0; cb < col_blocks; ++cb)
-    hipLaunchKernelGGL((expert_split_accumulate_kernel<DT, LPR>), dim3(blocks), dim3(kTokensPerBlock * kWave), 0, s,
+    hipLaunchKernelGGL((expert_split_accumulate_kernel<DT, LPR, true>), dim3(blocks), dim3(kTokensPerBlock * kWave), 0, s,
                        (const uint8_t*)down, gates, ids, partial, (uint8_t*)y, (int)T, H, k, (uint32_t)N, cb, col_blocks);
   return hipGetLastError();
 }
