@@ -637,7 +637,8 @@ __global__ __launch_bounds__(NW * 64, 1) void gemm_nt_dma_kernel(const GemmArgs 
 // memory before its first matrix instruction.  Ring loads are buffer loads (scalar base and tile offsets, one 32-bit
 // lane offset per operand).  The grid keeps every CU until the kernel ends, so a kernel on another stream finds no room
 // beside it: the callers use this form where nothing is meant to run concurrently.
-// Needs full tiles (M % 256 == 0, N a multiple of the tile's columns), K % 64 == 0, whole rounds of 256 tiles.
+// Needs N a multiple of the tile's columns and K % 64 == 0; a ragged last row tile re-reads the matrix's last row and stores
+// nothing for it.  XCD patches need whole rounds of 256 tiles; other tile counts go in plain order.
 //
 // The wave's 128 x 64 tile is 8 x 4 MFMA tiles of 16 x 16 and K advances 32 per instruction.  Under sustained load the
 // board clocks by power, and on the same operand bits the 16 x 16 x 32 instruction sustains about 15 % more than
@@ -667,7 +668,7 @@ __device__ __forceinline__ f32x4_t mfma16(const u32x4_t a, const u32x4_t b, f32x
   else return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
 }
 
-// Epilogue of the streaming kernel (full tiles, 16-byte stores).  Lanes l and l ^ 16 hold columns 4g..4g+3 and 4g+4..4g+7 of
+// Epilogue of the streaming kernel (full column tiles, 16-byte stores; rows past M are not stored).  Lanes l and l ^ 16 hold columns 4g..4g+3 and 4g+4..4g+7 of
 // two neighbouring column tiles: one v_permlane16_swap per word leaves every lane with 8 consecutive columns of one
 // of the two tiles, so each store instruction writes 64 consecutive bytes of 16 rows.
 template <int DT, int EPI>
@@ -696,7 +697,8 @@ __device__ __forceinline__ void stream_epilogue(const GemmArgs& g, f32x4_t (&acc
           }
         }
         if constexpr (EPI == kEpiResidual) {
-          const u32x2_t r = *(const u32x2_t*)(g.res + ((int64_t)m * g.N + nb + (j + t) * 16 + g4 * 4) * 2);
+          const int mr = m < g.M ? m : g.M - 1;          // rows past the matrix are exchanged but never stored
+          const u32x2_t r = *(const u32x2_t*)(g.res + ((int64_t)mr * g.N + nb + (j + t) * 16 + g4 * 4) * 2);
           const uint32_t r0 = r[0], r1 = r[1];
           if constexpr (DT == kBF16) {
             v[0] = Elem<DT>::round(v[0]) + bf16_lo(r0); v[1] = Elem<DT>::round(v[1]) + bf16_hi(r0);
@@ -713,7 +715,7 @@ __device__ __forceinline__ void stream_epilogue(const GemmArgs& g, f32x4_t (&acc
       const auto s0 = __builtin_amdgcn_permlane16_swap(w[0][0], w[1][0], false, false);
       const auto s1 = __builtin_amdgcn_permlane16_swap(w[0][1], w[1][1], false, false);
       const int n = nb + (j + (g4 & 1)) * 16 + (g4 & 2) * 4;
-      *(u32x4_t*)(g.c + ((int64_t)m * g.N + n) * 2) = u32x4_t{s0[0], s1[0], s0[1], s1[1]};
+      if (m < g.M) *(u32x4_t*)(g.c + ((int64_t)m * g.N + n) * 2) = u32x4_t{s0[0], s1[0], s0[1], s1[1]};
     }
   }
 }
@@ -741,7 +743,7 @@ __global__ __launch_bounds__(512, 1) void gemm_stream_kernel(const GemmArgs g) {
   // belongs at its (swizzled) position, which depends on the wave's parity and the lane only.  For the SwiGLU form rows
   // 64p .. 64p+31 of the weight tile are gate rows and 64p+32 .. 64p+63 the matching up rows of wave column p.
   const int sw = (lane & 7) ^ ((4 * (wave & 1) + (lane >> 4)) & 7);
-  const uint32_t a_voff = (uint32_t)(wave * 8 + (lane >> 3)) * row_bytes + sw * 16;
+  uint32_t a_voff[4];                                  // per load instruction: its row of the tile, clamped to the matrix (set with the cursor)
   const uint32_t b_voff = (uint32_t)((EPI == kEpiSwiglu ? (wave & 3) * 8 : wave * 8) + (lane >> 3)) * row_bytes + sw * 16;
   constexpr int kBRowsPerInstr = (EPI == kEpiSwiglu) ? 32 : 64;     // weight rows between consecutive load instructions of a wave
 
@@ -754,13 +756,16 @@ __global__ __launch_bounds__(512, 1) void gemm_stream_kernel(const GemmArgs g) {
     tile_coords_of(g, f_tile, tm, tn);
     f_a = (uint32_t)(tm * BM) * row_bytes;
     f_b = (uint32_t)(tn * BN) * row_bytes;
+    const int last = g.M - 1 - tm * BM;                // last row of the matrix, counted from the tile's first: a ragged last tile re-reads it
+#pragma unroll
+    for (int q = 0; q < 4; ++q) a_voff[q] = (uint32_t)min(q * 64 + wave * 8 + (lane >> 3), last) * row_bytes + sw * 16;
   };
   cursor_coords();
   auto issue_one = [&](int q) __attribute__((always_inline)) {       // q = 0..3: activation rows, 4..7: weight rows
     uint8_t* st = lds + f_stage * kStage;
     if (q < 4)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (__attribute__((address_space(3))) void*)(st + (8 * q + wave) * 1024), 16, a_voff,
-                                               f_a + (uint32_t)(q * 64) * row_bytes + f_kt * 128, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (__attribute__((address_space(3))) void*)(st + (8 * q + wave) * 1024), 16, a_voff[q],
+                                               f_a + f_kt * 128, 0, 0);
     else
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (__attribute__((address_space(3))) void*)(st + BM * kRow + (8 * (q - 4) + wave) * 1024), 16, b_voff,
                                                f_b + (uint32_t)((q - 4) * kBRowsPerInstr) * row_bytes + f_kt * 128, 0, 0);
@@ -1040,9 +1045,9 @@ static hipError_t launch_gemm(GemmArgs g, hipStream_t s) {
     constexpr int kDmaLds = kDmaStages * (BM + BR) * kDmaBK * 2;
     static_assert(kDmaLds <= 160 * 1024, "LDS ring exceeds 160 KiB");
     if constexpr (TM == 4 && TN == 4 && (EPI == kEpiPlain || EPI == kEpiSwiglu || EPI == kEpiResidual)) {
-      // full tiles in whole rounds of 256, K tiles enough for the two-stage prologue, nothing meant to run beside it: one
-      // block per CU streams through its tiles (buffer loads: operands below 1 Gi elements, 16-byte aligned)
-      const bool covers = g.exclusive && g.M % BM == 0 && g.N % BN == 0 && g.K >= 2 * kDmaBK && blocks % 256 == 0 && g.wide &&
+      // full column tiles, K tiles enough for the two-stage prologue, nothing meant to run beside it: one block per CU
+      // streams through its tiles (buffer loads: operands below 1 Gi elements, 16-byte aligned)
+      const bool covers = g.exclusive && g.N % BN == 0 && g.K >= 2 * kDmaBK && blocks >= 256 && g.wide &&
                           !g.save_gate && !(EPI != kEpiSwiglu && g.b1) && (int64_t)g.M * g.K < (1ll << 30) &&
                           (int64_t)g.N * g.K < (1ll << 30) && (uintptr_t)g.a % 16 == 0 && (uintptr_t)g.b0 % 16 == 0 &&
                           (EPI != kEpiSwiglu || (uintptr_t)g.b1 % 16 == 0);

@@ -21,7 +21,7 @@ def _ops():
 
 
 # the first four are the reference's benchmark grid (tests/test_mlp.py:144-150): intermediate 1024 .. 65536
-MLP_CASES = [(1024, 1024, 1024), (1024, 1024, 4096), (1024, 1024, 16384), (1024, 1024, 65536), (4096, 1024, 4096),
+MLP_CASES = [(1024, 1024, 1024), (1024, 1024, 4096), (1024, 1024, 16384), (1024, 1024, 65536), (4096, 1024, 4096), (4100, 1024, 4096),
              (333, 256, 1000), (128, 64, 128), (512, 2048, 8192), (5, 8, 8)]
 
 
@@ -407,7 +407,9 @@ LINEAR_CASES = [(3300, 1024, 512), (3300, 1024, 640), (3300, 1024, 576), (4096, 
                 (4096, 4096, 256), (300, 100, 264), (333, 1000, 256), (70, 4, 8),
                 (300, 62, 128), (129, 1001, 64), (70, 6, 16), (5, 1, 8),       # N % 4 != 0: element-wise stores
                 # few 64 x 64 tiles and K >= 512: the K tiles of a block dealt out over its waves (even and ragged shares, tails)
-                (4096, 128, 1024), (1000, 104, 512), (130, 72, 640), (64, 64, 4096), (200, 6, 576), (33, 250, 832)]
+                (4096, 128, 1024), (1000, 104, 512), (130, 72, 640), (64, 64, 4096), (200, 6, 576), (33, 250, 832),
+                # the streaming form with a ragged last row tile and with tile counts that are no whole rounds of 256
+                (4100, 4096, 512), (3328, 4096, 512), (4353, 4096, 128)]
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
