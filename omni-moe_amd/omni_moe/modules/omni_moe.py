@@ -98,12 +98,11 @@ class OmniMoE(nn.Module):
     # The fork and join cost about 50 us of host time per call, so below this much work (tokens x hidden x
     # intermediate; 2048 x 1024 x 4096 measured level on an MI355X) the call would be host-bound: one stream then.
     overlap_min_work = 2 ** 33
-    # ... and from this much work on, one stream is the faster schedule again: alone on the GPU the two big GEMMs take their
-    # streaming form (one block per CU walking its output tiles), which beats what the side branch gains beside them -- the
-    # chip is power-limited under the GEMMs, so overlapped kernels slow each other by about what they would cost alone
-    # (measured, hidden 1024 x intermediate 4096: 4096 tokens 134 against 143 us on two streams, 8192 tokens equal,
-    # 65536 tokens 1.85 against 1.70 ms; benchmark config 5: 3.58 against 3.43 ms).
-    overlap_max_work = 2 ** 35
+    # ... and from this much work on, one stream is the faster schedule again: the chip is power-limited under the GEMMs, so
+    # overlapped kernels slow each other by about what they would cost alone, and the fork and join are not free
+    # (measured, hidden 1024 x intermediate 4096, two streams against one: 4096 tokens 126 against 135 us, 8192 tokens 229
+    # against 241, 16384 tokens 425-440 against 415, 65536 tokens 1.66-1.70 against 1.63 ms; benchmark config 5: 3.43 against 3.17 ms).
+    overlap_max_work = 2 ** 36
     # Expert algorithm of the fused forward: "auto" decides from the sizes alone (no device-to-host read).  Which one is
     # faster also depends on how many DISTINCT experts the router picks: with tables far beyond the caches and a skewed
     # router (few live experts) "split" beats auto's "gather"; the caller who knows the distribution says so here.
