@@ -174,11 +174,11 @@ OMNI_API int32_t omni_swiglu_linear_fwd(const void* x, const void* gate_weight, 
 OMNI_API int32_t omni_linear_fwd(const void* x, const void* weight, const void* residual, void* y, int64_t num_tokens,
                                  int32_t in_features, int32_t out_features, int32_t dtype, void* stream);
 
-/* omni_swiglu_linear_fwd for callers that run other kernels beside it (another stream).  Where the product is whole rounds
- * of 256 x 256 tiles, omni_swiglu_linear_fwd / omni_linear_fwd / omni_mlp_fwd launch one block per CU that walks its share
- * of the tiles -- faster alone, but it holds every CU until it ends, so a concurrent kernel waits.  This entry never takes
- * that form (omni_moe_fwd with a side stream uses it for the gate/up projection).  Same results bit for bit.
- * No counterpart in the reference. */
+/* omni_swiglu_linear_fwd for callers that run other kernels beside it (another stream).  Where the product has at least 256
+ * tiles of 256 x 256, omni_swiglu_linear_fwd / omni_linear_fwd / omni_mlp_fwd launch one block per CU that walks its share
+ * of the tiles -- faster alone, but it holds every CU until it ends, so a concurrent kernel waits.  This entry launches one
+ * block per tile instead (omni_moe_fwd with a side stream uses it for a gate/up projection of at most two rounds of tiles).
+ * Same results bit for bit.  No counterpart in the reference. */
 OMNI_API int32_t omni_swiglu_linear_fwd_shared(const void* x, const void* gate_weight, const void* up_weight, void* h,
                                                int64_t num_tokens, int32_t hidden_size, int32_t intermediate_size,
                                                int32_t dtype, void* stream);

@@ -76,7 +76,7 @@ struct GemmArgs {           // all element offsets below are scaled by the eleme
   const float* gate;      // kEpiGate only: [M, N] fp32 factors; C is then [M, 2N]: round(v) in columns 0..N-1, round(v - round(v)) in N..2N-1
   uint8_t* save_gate;     // kEpiSwiglu only, or NULL: [M, N] the rounded gate and up projections, kept for a backward pass
   uint8_t* save_up;       //   (16-byte stores only: N % 8 == 0)
-  int exclusive;          // nothing is meant to run beside this launch: the 256 x 256 tile may take the streaming form, which holds every CU
+  int exclusive;          // nothing is meant to run beside this launch: the 256 x 256 tile's grid may be one block per CU that holds it to the end
 };
 
 // Which output tile a block owns.  Blocks go round-robin over the 8 XCDs; each XCD gets
@@ -1045,15 +1045,17 @@ static hipError_t launch_gemm(GemmArgs g, hipStream_t s) {
     constexpr int kDmaLds = kDmaStages * (BM + BR) * kDmaBK * 2;
     static_assert(kDmaLds <= 160 * 1024, "LDS ring exceeds 160 KiB");
     if constexpr (TM == 4 && TN == 4 && (EPI == kEpiPlain || EPI == kEpiSwiglu || EPI == kEpiResidual)) {
-      // full column tiles, K tiles enough for the two-stage prologue, nothing meant to run beside it: one block per CU
-      // streams through its tiles (buffer loads: operands below 1 Gi elements, 16-byte aligned)
-      const bool covers = g.exclusive && g.N % BN == 0 && g.K >= 2 * kDmaBK && blocks >= 256 && g.wide &&
+      // full column tiles, K tiles enough for the two-stage prologue (buffer loads: operands below 1 Gi elements, 16-byte
+      // aligned).  Nothing meant to run beside it: one block per CU streams through its tiles.  Otherwise the same kernel
+      // with one block per tile, so that CUs come free for the other stream's kernels as blocks retire (two-stream layer
+      // step at 4096 tokens, 1024 x 4096: 123.3 us against 127.2 us with the 32x32x16 kernel below in that place).
+      const bool covers = g.N % BN == 0 && g.K >= 2 * kDmaBK && blocks >= 256 && g.wide &&
                           !g.save_gate && !(EPI != kEpiSwiglu && g.b1) && (int64_t)g.M * g.K < (1ll << 30) &&
                           (int64_t)g.N * g.K < (1ll << 30) && (uintptr_t)g.a % 16 == 0 && (uintptr_t)g.b0 % 16 == 0 &&
                           (EPI != kEpiSwiglu || (uintptr_t)g.b1 % 16 == 0);
       if (covers) {
         if (hipError_t e = StreamKernelLds<DT, EPI>::entry.ensure(); e != hipSuccess) return e;
-        hipLaunchKernelGGL((gemm_stream_kernel<DT, EPI>), dim3(256), dim3(512), 2 * 512 * 128, s, g);
+        hipLaunchKernelGGL((gemm_stream_kernel<DT, EPI>), dim3(g.exclusive ? 256 : blocks), dim3(512), 2 * 512 * 128, s, g);
         return hipGetLastError();
       }
     }
