@@ -46,10 +46,10 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 # Bytes that cross the fabric per launch (FETCH_SIZE + WRITE_SIZE of rocprofv3 --pmc, each scaled by a plain copy of
 # known size); counters cannot be read in-process, so these are the figures of the committed summaries named here.
 TRAFFIC_SOURCE = ("profiles/bench_layer_c4_hbm_counters.txt, profiles/expert_c5_hbm_counters.txt; measured on the kernels as of the commit "
-                  "'GEMM: streaming form of the 256x256 tile' -- a later change to a kernel's memory access pattern needs a new counter run")
-TRAFFIC_BYTES = {"expert_c3": 180.6e6, "expert_c4": 57.8e6, "expert_gather_c3": 899.4e6, "gateup_c4": 134.5e6, "down_c4": 117.6e6,
-                 "down_plain_c4": 109.2e6, "schedule_c3": 12.36e6, "expert_segment_c3": 928.2e6, "expert_bwd_c3": 2159.4e6,
-                 "expert_c5_routed": 1029.2e6, "expert_c5_routed_split": 724.7e6, "expert_c5_uniform": 8846.8e6}
+                  "'Shared form of the 256x256 GEMM: the 16x16x32 kernel with one block per tile' -- a later change to a kernel's memory access pattern needs a new counter run")
+TRAFFIC_BYTES = {"expert_c3": 180.6e6, "expert_c4": 57.8e6, "expert_gather_c3": 899.6e6, "gateup_c4": 134.4e6, "down_c4": 117.6e6,
+                 "down_plain_c4": 109.2e6, "schedule_c3": 12.36e6, "expert_segment_c3": 928.1e6, "expert_bwd_c3": 2160.2e6,
+                 "expert_c5_routed": 1029.1e6, "expert_c5_routed_split": 724.9e6, "expert_c5_uniform": 8848.6e6}
 SECTIONS = ("layer", "kernels", "expert_c3", "expert_c5", "layer_c5", "ref_grid", "probe", "train", "cpu")
 
 
@@ -296,9 +296,9 @@ def main():
         h = hip.hip_swiglu_linear_func(xf, layer.gate_proj.weight, layer.up_proj.weight)
         y0 = hip.hip_linear_func(h, layer.down_proj.weight)
         r = layer.num_expert_sqrt
-        # the gate/up projection as the two-stream layer step runs it (a grid of 512 blocks that leaves room for the side branch) ...
+        # the gate/up projection as the two-stream layer step runs it (one block per tile: 512 blocks that leave room for the side branch as they retire) ...
         m, b = time_launches(torch, lambda: hip.hip_swiglu_linear_func(xf, layer.gate_proj.weight, layer.up_proj.weight, shared=True))
-        kernels.append(mfma_entry("gemm_nt_dma_kernel<swiglu> (gate/up projection + SwiGLU, as in the two-stream layer step), c4", 4 * T * H * I, m, b, TRAFFIC_BYTES["gateup_c4"], sustained))
+        kernels.append(mfma_entry("gemm_stream_kernel<swiglu>, one block per tile (gate/up projection + SwiGLU, as in the two-stream layer step), c4", 4 * T * H * I, m, b, TRAFFIC_BYTES["gateup_c4"], sustained))
         # ... and as every caller gets it that has the GPU to itself (operator calls, the one-stream layer): one block per CU streaming through its tiles
         m_s, b_s = time_launches(torch, lambda: hip.hip_swiglu_linear_func(xf, layer.gate_proj.weight, layer.up_proj.weight))
         kernels[-1]["streaming_form_alone_ms"] = m_s

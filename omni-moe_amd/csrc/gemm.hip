@@ -738,6 +738,8 @@ __global__ __launch_bounds__(512, 1) void gemm_stream_kernel(const GemmArgs g) {
   const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc((void*)g.a, 0, 0x7fffffff, 0x00020000);
   const uint8_t* bsel = (EPI == kEpiSwiglu && (wave >> 2)) ? g.b1 : g.b0;      // waves 0-3 fetch gate rows, 4-7 the up rows
   const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc((void*)bsel, 0, 0x7fffffff, 0x00020000);
+  // plain and residual forms: an optional second weight matrix supplies the upper half of the output columns (whole tiles of it)
+  const __amdgpu_buffer_rsrc_t rsrc_hi = __builtin_amdgcn_make_buffer_rsrc((void*)((EPI != kEpiSwiglu && g.b1) ? g.b1 : g.b0), 0, 0x7fffffff, 0x00020000);
 
   // Load instruction p of a wave fills LDS rows (8p + wave)*8 + lane/8 of a tile; the lane fetches the logical chunk that
   // belongs at its (swizzled) position, which depends on the wave's parity and the lane only.  For the SwiGLU form rows
@@ -751,11 +753,13 @@ __global__ __launch_bounds__(512, 1) void gemm_stream_kernel(const GemmArgs g) {
   int f_tile = blockIdx.x, f_kt = 0, f_stage = 0;
   bool half_pending = false;                          // the cursor's K tile has its activation half requested, not yet its weights
   uint32_t f_a = 0, f_b = 0;                          // byte offsets of the tile's first activation / weight row
+  bool f_hi = false;                                  // ... the weight row counted in the second weight matrix
   auto cursor_coords = [&]() {
     int tm, tn;
     tile_coords_of(g, f_tile, tm, tn);
     f_a = (uint32_t)(tm * BM) * row_bytes;
-    f_b = (uint32_t)(tn * BN) * row_bytes;
+    f_hi = EPI != kEpiSwiglu && g.b1 != nullptr && tn * BN >= g.N / 2;
+    f_b = (uint32_t)(tn * BN - (f_hi ? g.N / 2 : 0)) * row_bytes;
     const int last = g.M - 1 - tm * BM;                // last row of the matrix, counted from the tile's first: a ragged last tile re-reads it
 #pragma unroll
     for (int q = 0; q < 4; ++q) a_voff[q] = (uint32_t)min(q * 64 + wave * 8 + (lane >> 3), last) * row_bytes + sw * 16;
@@ -767,8 +771,8 @@ __global__ __launch_bounds__(512, 1) void gemm_stream_kernel(const GemmArgs g) {
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (__attribute__((address_space(3))) void*)(st + (8 * q + wave) * 1024), 16, a_voff[q],
                                                f_a + f_kt * 128, 0, 0);
     else
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (__attribute__((address_space(3))) void*)(st + BM * kRow + (8 * (q - 4) + wave) * 1024), 16, b_voff,
-                                               f_b + (uint32_t)((q - 4) * kBRowsPerInstr) * row_bytes + f_kt * 128, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(f_hi ? rsrc_hi : rsrc_b, (__attribute__((address_space(3))) void*)(st + BM * kRow + (8 * (q - 4) + wave) * 1024),
+                                               16, b_voff, f_b + (uint32_t)((q - 4) * kBRowsPerInstr) * row_bytes + f_kt * 128, 0, 0);
   };
   auto cursor_advance = [&]() {                        // after a K tile's second half has been issued
     f_stage ^= 1;
@@ -1050,9 +1054,9 @@ static hipError_t launch_gemm(GemmArgs g, hipStream_t s) {
       // with one block per tile, so that CUs come free for the other stream's kernels as blocks retire (two-stream layer
       // step at 4096 tokens, 1024 x 4096: 123.3 us against 127.2 us with the 32x32x16 kernel below in that place).
       const bool covers = g.N % BN == 0 && g.K >= 2 * kDmaBK && blocks >= 256 && g.wide &&
-                          !g.save_gate && !(EPI != kEpiSwiglu && g.b1) && (int64_t)g.M * g.K < (1ll << 30) &&
+                          !g.save_gate && (EPI == kEpiSwiglu || !g.b1 || (g.N / 2) % BN == 0) && (int64_t)g.M * g.K < (1ll << 30) &&
                           (int64_t)g.N * g.K < (1ll << 30) && (uintptr_t)g.a % 16 == 0 && (uintptr_t)g.b0 % 16 == 0 &&
-                          (EPI != kEpiSwiglu || (uintptr_t)g.b1 % 16 == 0);
+                          (!g.b1 || (uintptr_t)g.b1 % 16 == 0);
       if (covers) {
         if (hipError_t e = StreamKernelLds<DT, EPI>::entry.ensure(); e != hipSuccess) return e;
         hipLaunchKernelGGL((gemm_stream_kernel<DT, EPI>), dim3(g.exclusive ? 256 : blocks), dim3(512), 2 * 512 * 128, s, g);

@@ -432,6 +432,32 @@ def test_linear_matches_matmul(case, dtype, device):
     assert torch.equal(got_r, (got.float() + res.float()).to(dtype))
 
 
+# (M, columns per weight matrix, K): streaming kernel (second matrix = whole tiles), K tiles dealt out over the waves, ring kernel, staged kernel
+LINEAR2_CASES = [(8192, 512, 256), (16384, 256, 128), (1000, 52, 512), (3000, 200, 192), (300, 36, 40)]
+
+
+@pytest.mark.parametrize("case", LINEAR2_CASES, ids=lambda c: f"M{c[0]}-N2x{c[1]}-K{c[2]}")
+def test_linear_two_weight_matrices_equals_one(case, device):
+    """omni_linear2_fwd (the router projection's form: the upper half of the output columns comes from a second weight
+    matrix) gives bit for bit what omni_linear_fwd gives on the concatenated weights."""
+    from omni_moe.ops.hip import _lib
+    M, n, K = case
+    g = torch.Generator().manual_seed(M + n)
+    x = torch.randn(M, K, generator=g).bfloat16().to(device)
+    w_lo = (torch.randn(n, K, generator=g) * 0.05).bfloat16().to(device)
+    w_hi = (torch.randn(n, K, generator=g) * 0.05).bfloat16().to(device)
+    print(f"linear2 M={M} N=2x{n} K={K}", flush=True)
+    want = _ops().hip_linear_func(x, torch.cat([w_lo, w_hi], 0))
+    ref = (x.double() @ torch.cat([w_lo, w_hi], 0).double().t())
+    assert ((want.double() - ref).abs() <= 2.0 ** -8 * ref.abs() * 1.01 + 1e-4 * ref.abs().max()).all()
+    got = torch.empty(M, 2 * n, dtype=torch.bfloat16, device=device)
+    lib = _lib.load()
+    _lib.check(lib.omni_linear2_fwd(x.data_ptr(), w_lo.data_ptr(), w_hi.data_ptr(), got.data_ptr(), M, K, n,
+                                    _lib.DTYPE_CODE[torch.bfloat16], _lib.stream_ptr()), "omni_linear2_fwd")
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)
+
+
 @pytest.mark.parametrize("overlap", [True, False], ids=["two-streams", "one-stream"])
 def test_layer_is_graph_capturable(overlap, device):
     """The library only launches kernels and records/waits events, so a whole layer forward (fork and join
