@@ -271,23 +271,30 @@ def main():
         del src, dst
 
     kernels = []
-    sustained = None
+    sustained = sustained32 = None
     if "probe" in sections:
         # matrix-core rate with nothing else going on, on 8 KiB of the real activations: the clock that the board
         # sustains under its power limit depends on the operand bits, so this is the ceiling a GEMM on this data has
         lib = _lib.load()
         blocks, iters = 1024, 2048
-        sink = torch.empty(blocks * 256, device=dev, dtype=torch.float32)
+        sink = torch.empty(blocks * 512, device=dev, dtype=torch.float32)
         ops = dx.view(-1)[:4096].contiguous()
-        ms, best = time_launches(torch, lambda: _lib.check(lib.omni_probe_mfma(ops.data_ptr(), sink.data_ptr(), blocks, iters, _lib.stream_ptr()),
-                                                           "omni_probe_mfma"), n=3, reps=3, warmup=1)
-        sustained = blocks * 4 * iters * 16 * 32768 / (ms * 1e-3) / 1e12
         zeros = torch.zeros_like(ops)
-        ms0, _ = time_launches(torch, lambda: lib.omni_probe_mfma(zeros.data_ptr(), sink.data_ptr(), blocks, iters, _lib.stream_ptr()), n=3, reps=3, warmup=1)
-        out["mfma_probe"] = {"sustained_TFLOPs_on_activations": sustained, "sustained_TFLOPs_on_zeros": blocks * 4 * iters * 16 * 32768 / (ms0 * 1e-3) / 1e12,
+
+        def probe(fn, data, flop):
+            ms, _ = time_launches(torch, lambda: _lib.check(fn(data.data_ptr(), sink.data_ptr(), blocks, iters, _lib.stream_ptr()), "omni_probe_mfma"),
+                                  n=3, reps=3, warmup=1)
+            return flop / (ms * 1e-3) / 1e12
+        flop32, flop16 = blocks * 4 * iters * 16 * 32768, blocks * 8 * iters * 32 * 16384
+        sustained32 = probe(lib.omni_probe_mfma, ops, flop32)
+        sustained = probe(lib.omni_probe_mfma16, ops, flop16)       # the instruction of the 256 x 256 GEMM kernel
+        out["mfma_probe"] = {"sustained_TFLOPs_on_activations": sustained, "sustained_TFLOPs_on_zeros": probe(lib.omni_probe_mfma16, zeros, flop16),
+                             "sustained_TFLOPs_on_activations_32x32x16": sustained32,
+                             "sustained_TFLOPs_on_zeros_32x32x16": probe(lib.omni_probe_mfma, zeros, flop32),
                              "published_peak_TFLOPs": MFMA_BF16_PEAK_TFLOPS,
-                             "note": "v_mfma_f32_32x32x16_bf16 from registers only, 4 waves per CU, no memory traffic: what the matrix cores sustain "
-                                     "under the board's power limit; with realistic operand bits it is well below the published peak"}
+                             "note": "v_mfma_f32_16x16x32_bf16 (8 waves per CU) and v_mfma_f32_32x32x16_bf16 (4 waves per CU) from registers only, "
+                                     "no memory traffic: what the matrix cores sustain under the board's power limit; with realistic operand "
+                                     "bits it is well below the published peak, and the 16x16x32 instruction sustains more"}
 
     if "kernels" in sections:
         xf = dx.view(-1, H)
@@ -311,9 +318,9 @@ def main():
         m_lib, b_lib = time_launches(torch, lambda: torch.matmul(h, layer.down_proj.weight.t()))
         del wcat
         m, b = time_launches(torch, lambda: hip.hip_linear_func(h, layer.down_proj.weight, e_out))
-        kernels.append(mfma_entry("gemm_nt_dma_kernel<residual> (down projection + experts add), c4", 2 * T * H * I, m, b, TRAFFIC_BYTES["down_c4"], sustained))
+        kernels.append(mfma_entry("gemm_nt_dma_kernel<residual> (down projection + experts add), c4", 2 * T * H * I, m, b, TRAFFIC_BYTES["down_c4"], sustained32))
         m, b = time_launches(torch, lambda: hip.hip_linear_func(h, layer.down_proj.weight))
-        kernels.append(mfma_entry("gemm_nt_dma_kernel<plain> (down projection alone, as on the two-stream path), c4", 2 * T * H * I, m, b, TRAFFIC_BYTES["down_plain_c4"], sustained))
+        kernels.append(mfma_entry("gemm_nt_dma_kernel<plain> (down projection alone, as on the two-stream path), c4", 2 * T * H * I, m, b, TRAFFIC_BYTES["down_plain_c4"], sustained32))
         kernels[-1]["library_gemm_same_flops_ms"] = m_lib
         m, b = time_launches(torch, lambda: hip.hip_add_inplace_func(y0, e_out))
         kernels.append(hbm_entry("add_inplace_kernel (join of the two branches), c4", m, b, 3 * T * H * 2, resident_in_hbm=False,

@@ -198,6 +198,10 @@ OMNI_API int32_t omni_swiglu_linear_save_fwd(const void* x, const void* gate_wei
  * under its power limit depends on how many of them toggle).  sink: num_blocks * 256 floats, overwritten.
  * The caller times the launch; the benchmark prints the result beside the published peak. */
 OMNI_API int32_t omni_probe_mfma(const void* operands, float* sink, int32_t num_blocks, int32_t iters, void* stream);
+/* The same for v_mfma_f32_16x16x32_bf16, the instruction of the 256 x 256 GEMM kernel: num_blocks blocks of 8 waves each
+ * issue iters x 32 of them (iters * 32 * 16384 flop per wave).  sink: num_blocks * 512 floats, overwritten.  Under the
+ * board's power limit this instruction sustains more than the 32x32x16 one on the same operand bits. */
+OMNI_API int32_t omni_probe_mfma16(const void* operands, float* sink, int32_t num_blocks, int32_t iters, void* stream);
 
 /* y[i] = round(y[i] + addend[i]) in place: the layer's final  mlp + experts  (omni_moe.py:102) as a
  * call of its own, for callers that run the two branches on different streams.  num_elements a

@@ -1355,7 +1355,42 @@ __global__ __launch_bounds__(kGemmThreads, 1) void mfma_probe_kernel(const u32x4
   for (int i = 0; i < 16; ++i) s += acc[i][0] + acc[i][5];
   sink[blockIdx.x * kGemmThreads + threadIdx.x] = s;
 }
+// The same with v_mfma_f32_16x16x32_bf16, the streaming kernel's instruction: 8 waves per block (two per SIMD, as that
+// kernel runs), 8 x 4 independent accumulator tiles per wave.
+__global__ __launch_bounds__(512, 1) void mfma_probe16_kernel(const u32x4_t* __restrict__ operands, float* __restrict__ sink, int iters) {
+  f32x4_t acc[8][4];
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) acc[i][j][q] = 0.f;
+  u32x4_t a[8], b[4];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) a[i] = operands[(threadIdx.x * 12 + i) & 511];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) b[i] = operands[(threadIdx.x * 12 + 8 + i) & 511];
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[i][j] = mfma16<kBF16>(b[j], a[i], acc[i][j]);
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) s += acc[i][j][0] + acc[i][j][3];
+  sink[blockIdx.x * 512 + threadIdx.x] = s;
+}
 }  // namespace omni
+
+extern "C" OMNI_API int32_t omni_probe_mfma16(const void* operands, float* sink, int32_t num_blocks, int32_t iters, void* stream) {
+  if (num_blocks <= 0 || iters <= 0) return OMNI_ERR_SHAPE;
+  if (!operands || !sink) return OMNI_ERR_NULL;
+  hipLaunchKernelGGL(omni::mfma_probe16_kernel, dim3(num_blocks), dim3(512), 0, (hipStream_t)stream, (const omni::u32x4_t*)operands, sink, iters);
+  return omni::to_code(hipGetLastError());
+}
 
 extern "C" OMNI_API int32_t omni_probe_mfma(const void* operands, float* sink, int32_t num_blocks, int32_t iters, void* stream) {
   if (num_blocks <= 0 || iters <= 0) return OMNI_ERR_SHAPE;

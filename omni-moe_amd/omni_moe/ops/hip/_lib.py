@@ -45,6 +45,7 @@ SIGNATURES = {
     "omni_moe_fwd_algo": (c_int32, [c_void_p] * 15 + [c_int64, c_int32, c_int32, c_int64, c_int32, c_int32, c_int32, c_int32,
                                     c_int32, c_float, c_float] + [c_void_p] * 5 + [c_int32]),
     "omni_probe_mfma": (c_int32, [c_void_p, c_void_p, c_int32, c_int32, c_void_p]),
+    "omni_probe_mfma16": (c_int32, [c_void_p, c_void_p, c_int32, c_int32, c_void_p]),
     "omni_add_inplace": (c_int32, [c_void_p, c_void_p, c_int64, c_int32, c_void_p]),
     "omni_linear2_fwd": (c_int32, [c_void_p] * 4 + [c_int64, c_int32, c_int32, c_int32, c_void_p]),
     "omni_router_workspace_bytes": (c_size_t, [c_int64, c_int32, c_int32]),
