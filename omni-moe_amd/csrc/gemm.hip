@@ -716,6 +716,26 @@ __device__ __forceinline__ void stream_epilogue(const GemmArgs& g, f32x4_t (&acc
       const auto s1 = __builtin_amdgcn_permlane16_swap(w[0][1], w[1][1], false, false);
       const int n = nb + (j + (g4 & 1)) * 16 + (g4 & 2) * 4;
       if (m < g.M) *(u32x4_t*)(g.c + ((int64_t)m * g.N + n) * 2) = u32x4_t{s0[0], s1[0], s0[1], s1[1]};
+      if constexpr (EPI == kEpiSwiglu) {
+        if (g.save_gate) {                               // the two rounded projections leave the same way (kept for a backward pass)
+          uint32_t a[2][2], b[2][2];
+#pragma unroll
+          for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int h2 = 0; h2 < 2; ++h2) {
+              a[t][h2] = pack2<DT>(acc[i][j + t][2 * h2], acc[i][j + t][2 * h2 + 1]);
+              b[t][h2] = pack2<DT>(acc[i][j + t + TNO][2 * h2], acc[i][j + t + TNO][2 * h2 + 1]);
+            }
+          const auto a0 = __builtin_amdgcn_permlane16_swap(a[0][0], a[1][0], false, false);
+          const auto a1 = __builtin_amdgcn_permlane16_swap(a[0][1], a[1][1], false, false);
+          const auto b0 = __builtin_amdgcn_permlane16_swap(b[0][0], b[1][0], false, false);
+          const auto b1 = __builtin_amdgcn_permlane16_swap(b[0][1], b[1][1], false, false);
+          if (m < g.M) {
+            *(u32x4_t*)(g.save_gate + ((int64_t)m * g.N + n) * 2) = u32x4_t{a0[0], a1[0], a0[1], a1[1]};
+            *(u32x4_t*)(g.save_up + ((int64_t)m * g.N + n) * 2) = u32x4_t{b0[0], b1[0], b0[1], b1[1]};
+          }
+        }
+      }
     }
   }
 }
@@ -1054,7 +1074,7 @@ static hipError_t launch_gemm(GemmArgs g, hipStream_t s) {
       // with one block per tile, so that CUs come free for the other stream's kernels as blocks retire (two-stream layer
       // step at 4096 tokens, 1024 x 4096: 123.3 us against 127.2 us with the 32x32x16 kernel below in that place).
       const bool covers = g.N % BN == 0 && g.K >= 2 * kDmaBK && blocks >= 256 && g.wide &&
-                          !g.save_gate && (EPI == kEpiSwiglu || !g.b1 || (g.N / 2) % BN == 0) && (int64_t)g.M * g.K < (1ll << 30) &&
+                          (EPI == kEpiSwiglu || !g.b1 || (g.N / 2) % BN == 0) && (int64_t)g.M * g.K < (1ll << 30) &&
                           (int64_t)g.N * g.K < (1ll << 30) && (uintptr_t)g.a % 16 == 0 && (uintptr_t)g.b0 % 16 == 0 &&
                           (!g.b1 || (uintptr_t)g.b1 % 16 == 0);
       if (covers) {
