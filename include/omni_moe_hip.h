@@ -75,7 +75,8 @@ OMNI_API int32_t omni_init(void);
  *   indices            : device [num_tokens, k] int32, ix*num_expert_sqrt+iy
  * Contract of utils.py:81-104: 0 <= k <= r*r, k <= 128, k even (else OMNI_ERR_TOPK).
  * Ties: the lower key index wins inside a half; the lower candidate position
- * a*k'+b (a, b = ranks in the two halves, k' = min(r,k)) wins among equal sums. */
+ * a*k'+b (a, b = ranks in the two halves, k' = min(r,k)) wins among equal sums.
+ * num_expert_sqrt <= 1024; with bf16/f16 scores and k <= 64 up to 16384 (else OMNI_ERR_UNSUPPORTED). */
 OMNI_API int32_t omni_router_select(const void* logits_x, const void* logits_y, void* scores, int32_t* indices,
                            int64_t num_tokens, int32_t num_expert_sqrt, int32_t num_experts_per_token,
                            int32_t dtype, void* stream);
@@ -285,7 +286,9 @@ OMNI_API int32_t omni_linear2_fwd(const void* x, const void* weight_lo, const vo
  *     average with factor 1 / num_batches_tracked (the counters are then required); one token in
  *     training is OMNI_ERR_SHAPE (nn.BatchNorm1d raises).  training == 0: the buffers
  *     normalise, nothing is written.
- *   Limits (OMNI_ERR_UNSUPPORTED, nothing enqueued): num_expert_sqrt > 1024; and training with
+ *   Limits (OMNI_ERR_UNSUPPORTED, nothing enqueued): num_expert_sqrt > 1024 with fp32 scores or k > 64, and
+ *     num_expert_sqrt > 16384 (up to 1024 keys per half the selection holds the row in registers; beyond that it
+ *     walks the row in chunks, with 16-bit scores and at most 64 candidates per half); and training with
  *     momentum < 0 and k == 0 (no selection follows the statistics, and the cumulative average's
  *     counter is advanced by the selection kernel).
  *   gates [T,k] dtype = exp(score); indices [T,k] int32; scores [T,k] dtype or NULL

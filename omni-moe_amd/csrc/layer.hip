@@ -11,6 +11,8 @@ static inline size_t up256(size_t v) { return (v + 255) / 256 * 256; }
 static inline size_t elem_bytes(int dtype) { return dtype == OMNI_F32 ? 4 : 2; }
 // defined beside the expert kernels: OMNI_OK when omni_expert_fwd takes `algo` at this shape (decided from the sizes alone)
 int expert_algo_check(int algo, int64_t num_tokens, int hidden_size, int64_t num_experts, int top_k, int dtype);
+// defined beside the select kernels: whether they take num_expert_sqrt keys per half with top_k and this dtype
+bool select_covers(int r, int k, int dtype);
 // defined beside the GEMM kernels: omni_linear_fwd with the caller's word on whether the launch has the GPU to itself
 // (then a GEMM of whole 256-tile rounds may take the form that holds every CU until it ends)
 int linear_fwd_impl(const void* x, const void* weight, const void* residual, void* y, int64_t num_tokens, int32_t in_features,
@@ -70,7 +72,7 @@ extern "C" OMNI_API int32_t omni_moe_fwd_algo(const void* x, const void* gate_we
     const int64_t esz = (int64_t)elem_bytes(dtype), r = num_expert_sqrt, k = num_experts_per_token;
     if ((hidden_size * esz) % 16 != 0 || (intermediate_size * esz) % 16 != 0) return OMNI_ERR_SHAPE;   // rows are fetched 16 bytes at a time
     if (k < 0 || k > r * r || k > 128 || k % 2 != 0) return OMNI_ERR_TOPK;
-    if (r > 1024) return OMNI_ERR_UNSUPPORTED;
+    if (!select_covers((int)r, (int)k, dtype)) return OMNI_ERR_UNSUPPORTED;
     if (r * r > num_experts) return OMNI_ERR_SHAPE;                                                   // ids reach r*r - 1
     if (int e = expert_algo_check(expert_algo, num_tokens, hidden_size, num_experts, num_experts_per_token, dtype)) return e;
   }

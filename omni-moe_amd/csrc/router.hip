@@ -198,7 +198,8 @@ __device__ __forceinline__ void store_score(void* p, int64_t i, float v, int dt)
 }
 
 constexpr int kRouterWaves = 4;
-constexpr int kMaxKeys = 1024;        // keys per half that the select kernels hold (16 per lane)
+constexpr int kMaxKeys = 1024;        // keys per half that the select kernels hold in registers (16 per lane)
+constexpr int kMaxKeysChunked = 16384; // ... that the chunked kernel walks (16-bit scores, at most 64 candidates per half)
 constexpr float kNegInf = -__builtin_huge_valf();
 
 struct SelectArgs {
@@ -233,6 +234,19 @@ __device__ __forceinline__ void count_batch(const SelectArgs& g) {
       g.stats_out[(2 * half + 1) * g.r + key] = __builtin_amdgcn_rsqf(load_score(g.run_var[half], key, g.stat_dt) + g.eps);
     }
   }
+}
+
+// BatchNorm (affine-free) of one raw projection value, rounded to the storage dtype as the reference's BatchNorm output is
+__device__ __forceinline__ float normalise_one(float v, const SelectArgs& g, const int half, const int key, const int r, const int dt) {
+  float mean, rstd;
+  if (g.stats) {
+    mean = g.stats[(2 * half) * r + key];
+    rstd = g.stats[(2 * half + 1) * r + key];
+  } else {
+    mean = load_score(g.run_mean[half], key, g.stat_dt);
+    rstd = __builtin_amdgcn_rsqf(load_score(g.run_var[half], key, g.stat_dt) + g.eps);
+  }
+  return round_score((v - mean) * rstd, dt);
 }
 
 // BatchNorm (affine-free) then log-softmax of one half, in place: v holds the raw projection
@@ -582,6 +596,114 @@ __global__ __launch_bounds__(kRouterWaves* kWave) void router_select_packed_kern
   }
 }
 
+// More keys per half than a wave's registers hold (r > 1024): 16-bit scores, k' <= 64.  The row is walked in chunks of
+// 512 keys per half: each chunk's 64 best (ktop64_2) are merged into the running 64 best by the same max(A[i], B[63-i])
+// step.  With the BatchNorm + log-softmax front the row is read three times (maximum, sum of exponentials, keys), each
+// time with the arithmetic and the per-lane summation order of normalise_half, so a row gives the bits it would give there.
+template <int C>
+__global__ __launch_bounds__(kRouterWaves* kWave) void router_select_chunked_kernel(const SelectArgs g) {
+  constexpr int RC = 8, kChunk = RC * kWave;
+  count_batch(g);
+  const int lane = lane_id();
+  const int wave = blockIdx.x * kRouterWaves + (threadIdx.x >> 6);
+  const int num_waves = gridDim.x * kRouterWaves;
+  const int r = g.r, k = g.k, kp = g.kp, dt = g.dt;
+  const int chunks = (r + kChunk - 1) / kChunk;
+  const bool norm = g.stats || g.run_mean[0];
+  int cell[C];
+  candidate_cells<1, C>(cell, g, kp, lane);
+
+  for (int t = wave; t < g.num_tokens; t += num_waves) {
+    const int64_t row = int64_t(t) * g.row_stride;
+    float mx[2] = {0.f, 0.f}, lse[2] = {0.f, 0.f};
+    if (norm) {
+      for (int half = 0; half < 2; ++half) {
+        const void* src = half ? g.ly : g.lx;
+        float m = kNegInf;
+        for (int c = 0; c < chunks; ++c)
+#pragma unroll
+          for (int a = 0; a < RC; ++a) {
+            const int key = c * kChunk + a * kWave + lane;
+            if (key < r) m = fmaxf(m, normalise_one(load_score(src, row + key, dt), g, half, key, r, dt));
+          }
+        m = wave_max(m);
+        float e = 0.f;
+        for (int c = 0; c < chunks; ++c)
+#pragma unroll
+          for (int a = 0; a < RC; ++a) {
+            const int key = c * kChunk + a * kWave + lane;
+            e += key < r ? expf(normalise_one(load_score(src, row + key, dt), g, half, key, r, dt) - m) : 0.f;
+          }
+        mx[half] = m;
+        lse[half] = logf(wave_sum(e));
+      }
+    }
+    uint32_t bx = 0u, by = 0u;                      // the 64 best keys so far of each half, descending across the lanes
+    for (int c = 0; c < chunks; ++c) {
+      uint32_t kx[RC], ky[RC];
+#pragma unroll
+      for (int a = 0; a < RC; ++a) {
+        const int key = c * kChunk + a * kWave + lane;
+        const bool ok = key < r;
+        float vx = ok ? load_score(g.lx, row + key, dt) : 0.f, vy = ok ? load_score(g.ly, row + key, dt) : 0.f;
+        if (norm && ok) {
+          vx = round_score(normalise_one(vx, g, 0, key, r, dt) - mx[0] - lse[0], dt);
+          vy = round_score(normalise_one(vy, g, 1, key, r, dt) - mx[1] - lse[1], dt);
+        }
+        kx[a] = ok ? make_key(vx, key, dt) : 0u;    // 0 sorts behind every real key
+        ky[a] = ok ? make_key(vy, key, dt) : 0u;
+      }
+      ktop64_2<RC>(kx, ky, lane);
+      uint32_t x[1] = {max(bx, (uint32_t)__shfl((int)kx[0], 63 - lane, kWave))};
+      uint32_t y[1] = {max(by, (uint32_t)__shfl((int)ky[0], 63 - lane, kWave))};
+      kstages_ct<1, kWave, kWave / 2>(x, y, lane, true);
+      bx = c == 0 ? kx[0] : x[0];
+      by = c == 0 ? ky[0] : y[0];
+    }
+    const uint32_t sx[1] = {bx}, sy[1] = {by};
+
+    uint32_t ck[C];
+#pragma unroll
+    for (int c = 0; c < C; ++c) {
+      const bool ok = cell[c] >= 0;
+      const int a = ok ? (cell[c] >> 8) : 0, b = ok ? (cell[c] & 255) : 0;
+      const float va = key_score(sorted_key<1>(sx, a), dt), vb = key_score(sorted_key<1>(sy, b), dt);
+      ck[c] = ok ? make_key(round_score(va + vb, dt), cell[c], dt) : 0u;
+    }
+    ksort<C>(ck, lane);
+
+    constexpr int kOut = (C >= 2) ? 2 : 1;
+#pragma unroll
+    for (int c = 0; c < kOut; ++c) {
+      const int j = c * kWave + lane;
+      const bool ok = j < k;
+      const int pl = ok ? key_payload(ck[c]) : 0;
+      const int ia = key_payload(sorted_key<1>(sx, pl >> 8)), ib = key_payload(sorted_key<1>(sy, pl & 255));
+      if (ok) {
+        const int64_t o = int64_t(t) * k + j;
+        const float sc = key_score(ck[c], dt);
+        if (g.scores) store_score(g.scores, o, sc, dt);
+        if (g.gates) store_score(g.gates, o, expf(sc), dt);
+        g.indices[o] = ia * r + ib;
+      }
+    }
+  }
+}
+
+template <int C>
+static hipError_t launch_select_chunked(const SelectArgs& g, hipStream_t s) {
+  int64_t blocks = ((int64_t)g.num_tokens + kRouterWaves - 1) / kRouterWaves;
+  if (blocks > 256 * 16) blocks = 256 * 16;
+  hipLaunchKernelGGL((router_select_chunked_kernel<C>), dim3((unsigned)blocks), dim3(kRouterWaves * kWave), 0, s, g);
+  return hipGetLastError();
+}
+
+// What the select kernels take: r <= 1024 with every dtype and k <= 128; beyond that 16-bit scores with k <= 64.
+bool select_covers(int r, int k, int dtype) {
+  if (r <= kMaxKeys) return true;
+  return r <= kMaxKeysChunked && dtype != kF32 && k <= kWave;
+}
+
 static int num_cells(int k, int kp) {
   int n = 0;
   for (int a = 0; a < kp; ++a) n += (kp < k / (a + 1)) ? kp : k / (a + 1);
@@ -619,7 +741,11 @@ static int select_dispatch(SelectArgs g, hipStream_t s) {
   else if (rpl <= 4) err = select_by_cells<4>(cpl, g, s);
   else if (rpl <= 8) err = select_by_cells<8>(cpl, g, s);
   else if (rpl <= 16) err = select_by_cells<16>(cpl, g, s);
-  else return OMNI_ERR_UNSUPPORTED;                          // r > kMaxKeys: the entry points refuse it before anything is enqueued
+  else if (!select_covers(g.r, g.k, g.dt)) return OMNI_ERR_UNSUPPORTED;   // the entry points refuse it before anything is enqueued
+  else if (cpl <= 1) err = launch_select_chunked<1>(g, s);
+  else if (cpl <= 2) err = launch_select_chunked<2>(g, s);
+  else if (cpl <= 4) err = launch_select_chunked<4>(g, s);
+  else err = launch_select_chunked<8>(g, s);                // k <= 64: at most 280 cells
   return err == hipSuccess ? OMNI_OK : OMNI_ERR_HIP_BASE + (int)err;
 }
 
@@ -703,7 +829,7 @@ extern "C" OMNI_API int32_t omni_router_select(const void* logits_x, const void*
   if (dtype != OMNI_BF16 && dtype != OMNI_F16 && dtype != OMNI_F32) return OMNI_ERR_DTYPE;
   if (num_tokens == 0 || k == 0) return OMNI_OK;
   if (!logits_x || !logits_y || !scores || !indices) return OMNI_ERR_NULL;
-  if (r > kMaxKeys) return OMNI_ERR_UNSUPPORTED;
+  if (!select_covers(r, k, dtype)) return OMNI_ERR_UNSUPPORTED;
   SelectArgs g{};
   g.lx = logits_x; g.ly = logits_y; g.row_stride = r; g.scores = scores; g.indices = indices;
   g.num_tokens = (int)num_tokens; g.r = r; g.k = k; g.dt = dtype;
@@ -746,7 +872,7 @@ extern "C" OMNI_API int32_t omni_router_fwd(const void* x, const void* weight_x,
   if (!x || !weight_x || !weight_y || !running_mean_x || !running_var_x || !running_mean_y || !running_var_y) return OMNI_ERR_NULL;
   if (training && momentum < 0.f && (!num_batches_tracked_x || !num_batches_tracked_y)) return OMNI_ERR_NULL;   // the cumulative average needs the counts
   if (training && momentum < 0.f && k == 0) return OMNI_ERR_UNSUPPORTED;
-  if (r > kMaxKeys) return OMNI_ERR_UNSUPPORTED;           // the select kernels' limit, checked before the projection is enqueued
+  if (k > 0 && !select_covers(r, k, dtype)) return OMNI_ERR_UNSUPPORTED;   // the select kernels' limit, checked before the projection is enqueued
   if (k > 0 && (!gates || !indices)) return OMNI_ERR_NULL;
   if (!workspace) return OMNI_ERR_WORKSPACE;
   hipStream_t s = (hipStream_t)stream;

@@ -87,8 +87,10 @@ def test_argument_errors_need_no_gpu():
     assert lib.omni_router_fwd(*([p] * 9), 1, 0.1, 1e-5, p, p, None, 1, 64, 4, 2, 0, 2, p, None) == -2
     assert lib.omni_router_fwd(p, p, p, p, p, None, p, p, None, 1, -1.0, 1e-5, p, p, None, 4, 64, 4, 2, 0, 2, p, None) == -1   # cumulative average needs the counters
     # limits of the select kernels and of the schedule's multiply-shift division: refused before anything is enqueued
-    assert lib.omni_router_fwd(*([p] * 9), 0, 0.1, 1e-5, p, p, None, 4, 64, 1025, 2, 0, 2, p, None) == -5      # r > 1024
-    assert lib.omni_router_select(p, p, p, p, 4, 1025, 2, 0, None) == -5
+    assert lib.omni_router_fwd(*([p] * 9), 0, 0.1, 1e-5, p, p, None, 4, 64, 1025, 2, 2, 2, p, None) == -5      # r > 1024 with fp32 scores
+    assert lib.omni_router_fwd(*([p] * 9), 0, 0.1, 1e-5, p, p, None, 4, 64, 1025, 66, 0, 2, p, None) == -5     # r > 1024 with k > 64
+    assert lib.omni_router_select(p, p, p, p, 4, 1025, 2, 2, None) == -5
+    assert lib.omni_router_select(p, p, p, p, 4, 16385, 2, 0, None) == -5                                       # r > 16384
     assert lib.omni_schedule(p, p, p, p, 1 << 20, 1024, 16, p, None) == -2                                      # 2^30 pairs
     import torch
     if not torch.cuda.is_available():

@@ -68,7 +68,7 @@ def test_mlp_fp32_matches_oracle(case, device):
 
 # the last two make the projection GEMM pick its 128 x 128 and 256 x 256 tiles (statistics epilogue included)
 ROUTER_FWD_CASES = [(4096, 1024, 64, 16), (1024, 256, 32, 8), (2048, 2048, 512, 32), (300, 520, 36, 10), (300, 576, 36, 10),
-                    (4096, 256, 512, 32), (16384, 256, 512, 32)]
+                    (4096, 256, 512, 32), (16384, 256, 512, 32), (200, 128, 1300, 16)]      # last: more than 1024 keys per half
 
 
 def _bn_buffers(r, dtype, device=None):
@@ -148,6 +148,7 @@ LAYER_CASES = [
     (300, 128, 256, 1000, 8, 1),       # N not a square: r = floor(sqrt(N)) = 31 (omni_moe.py:38), odd, ids < 961
     (300, 128, 256, 1000, 40, 1),      # and k > r, so k' = r
     (64, 64, 128, 50, 6, 2),           # r = 7
+    (200, 64, 128, 1100 * 1100, 8, 4), # r = 1100: more keys per half than the select kernels hold in registers
 ]
 
 

@@ -35,7 +35,12 @@ ROUTER_CASES = [
     (64, 4, 16, torch.bfloat16, "randn"),          # k = r*r: every expert selected, k' = r
     (64, 8, 32, torch.float32, "randn"),           # k > r
     (100, 128, 128, torch.bfloat16, "randn"),      # largest k the contract allows
-    (100, 1024, 64, torch.bfloat16, "randn"),      # largest r the kernel covers
+    (100, 1024, 64, torch.bfloat16, "randn"),      # largest r the kernels hold in registers
+    (70, 1025, 2, torch.bfloat16, "randn"),        # beyond: the row is walked in chunks of 512 keys (16-bit scores, k <= 64)
+    (50, 1500, 16, torch.bfloat16, "logprob"),
+    (40, 2048, 64, torch.float16, "randn"),
+    (30, 4096, 32, torch.bfloat16, "ties"),
+    (9, 16384, 8, torch.bfloat16, "randn"),
     (512, 64, 16, torch.bfloat16, "ties"),         # heavy ties: scores on a coarse grid
     (512, 64, 16, torch.float32, "allequal"),      # all scores equal: pure tie-break
     (1, 64, 2, torch.bfloat16, "randn"),
