@@ -778,6 +778,9 @@ __global__ __launch_bounds__(256) void bn_finalize_kernel(const BnFinalArgs g) {
   const int half = col >= g.r, key = col - half * g.r;
   float mean, var;
   if (g.training) {
+    // the running buffers (and the batch count) are requested first: their latency passes beside the strips'
+    const float rm = load_score(g.running_mean[half], key, g.stat_dt), rv = load_score(g.running_var[half], key, g.stat_dt);
+    const float f = g.momentum >= 0.f ? g.momentum : 1.0f / (float)(*g.num_batches_tracked[half] + 1);
     // one pass over the strips, both sums in double: M2 = sum (M2_s + n_s mean_s^2) - n mu^2 (double carries 29 bits more than
     // the fp32 result keeps, so the difference stays exact to fp32 while mean^2 / variance < 2^29)
     double wsum = 0., q = 0.;
@@ -799,9 +802,7 @@ __global__ __launch_bounds__(256) void bn_finalize_kernel(const BnFinalArgs g) {
     var = (float)(m2 / n);                                   // biased: normalises the batch
     if (lane == 0) {
       const float unbiased = (float)(m2 / (n > 1. ? n - 1. : 1.));
-      const float rm = load_score(g.running_mean[half], key, g.stat_dt), rv = load_score(g.running_var[half], key, g.stat_dt);
-      // nn.BatchNorm1d(momentum=None): the factor is 1 / num_batches_tracked AFTER this batch has been counted
-      const float f = g.momentum >= 0.f ? g.momentum : 1.0f / (float)(*g.num_batches_tracked[half] + 1);
+      // nn.BatchNorm1d(momentum=None): the factor f is 1 / num_batches_tracked AFTER this batch has been counted
       store_score(g.running_mean[half], key, (1.f - f) * rm + f * mean, g.stat_dt);
       store_score(g.running_var[half], key, (1.f - f) * rv + f * unbiased, g.stat_dt);
     }
