@@ -438,16 +438,18 @@ def main():
                                  note="same inputs as the entry above, algo='split' by name (OmniMoE.expert_algo = 'split'): the live rows' column slices fit the XCDs' L2s"))
         m_a, b_a = time_launches(torch, lambda: hip.hip_omni_expert_func(x5, up5, down5, g5, i5), n=10, reps=5, warmup=2)
         out["expert_c5_routed"] = {"gather_ms": m, "split_ms": m_s, "auto_ms": m_a, "distinct_experts": used, "max_pairs_per_expert": int(counts.max()),
-                                   "note": "AUTO decides by table size (2 GiB: gather); the layer takes a hint (OmniMoE.expert_algo) where the id distribution is known"}
+                                   "note": "AUTO decides from the sizes alone (512-byte row slices and a million pairs: split); the layer takes a hint (OmniMoE.expert_algo) where the caller knows better"}
         # the same shape with ids spread evenly (32 distinct experts per token, uniform over all 262144): every selected
         # row comes from HBM, so algorithmic bytes are HBM bytes -- the case that shows the kernel against the HBM roofline
         iu = torch.randint(0, N5 // k5, (T5, k5), device=dev, generator=g, dtype=torch.int32) * k5 + torch.arange(k5, device=dev, dtype=torch.int32)
-        yu = hip.hip_omni_expert_func(x5, up5, down5, g5, iu)
+        yu = hip.hip_omni_expert_func(x5, up5, down5, g5, iu, algo="gather")
         check5(yu, g5, iu)
-        m, b = time_launches(torch, lambda: hip.hip_omni_expert_func(x5, up5, down5, g5, iu), n=10, reps=5, warmup=2)
+        m, b = time_launches(torch, lambda: hip.hip_omni_expert_func(x5, up5, down5, g5, iu, algo="gather"), n=10, reps=5, warmup=2)
+        m_us, _ = time_launches(torch, lambda: hip.hip_omni_expert_func(x5, up5, down5, g5, iu, algo="split"), n=10, reps=5, warmup=2)
         e5 = hbm_entry("expert op (gather algorithm: expert_gather_kernel), config-5 shape (32768 tokens, hidden 2048, 262144 experts, top-32), ids uniform over the experts",
                        m, b, alg5, TRAFFIC_BYTES["expert_c5_uniform"], 2 * T5 * H5 * 2 + 2 * torch.unique(iu).numel() * H5 * 2 + T5 * k5 * 6, resident_in_hbm=True,
                        note="2 GiB of tables, no reuse to speak of: the rocprofv3 byte counters of this launch read the algorithmic bytes (profiles/expert_c5_hbm_counters.txt)")
+        e5["split_algorithm_same_ids_ms"] = m_us            # what AUTO runs at this shape; no byte counters were taken for it
         kernels.append(e5)
         out["roofline_expert_hbm"] = e5
         del y5, ys, iu, yu
@@ -464,7 +466,7 @@ def main():
         # the 2 GiB tables are the ones drawn above: the module's parameters alias them (no second copy in HBM)
         layer5.up_embed.weight.data, layer5.down_embed.weight.data = up5, down5
         per_algo = {}
-        for algo in ("auto", "split"):
+        for algo in ("auto", "gather"):                 # AUTO takes the split algorithm at this shape
             layer5.expert_algo = algo
             y5l = layer5(x5.view(8, T5 // 8, H5)).view(T5, H5)
             # oracle on a token subset (eval mode is token-independent): router ids, then experts over the selected rows + MLP
@@ -506,7 +508,7 @@ def main():
         out["layer_c5"] = {"workload": "BASELINE.json configs[4] (benchmark config 5): full OmniMoE layer forward, 8x4096 tokens, hidden 2048, intermediate 8192, "
                                        "262144 experts (512x512), top-32, eval-mode BatchNorm whose buffers carry the Zipf(1.1) key bias, seed 4",
                            "ms_per_step": per_algo["auto"]["ms_per_step"], "tokens_per_s": per_algo["auto"]["tokens_per_s"],
-                           "with_expert_algo_split": per_algo["split"], "on_two_streams": {"ms_per_step": m2, "ms_per_step_best": b2},
+                           "with_expert_algo_gather": per_algo["gather"], "on_two_streams": {"ms_per_step": m2, "ms_per_step_best": b2},
                            "router_stage_ms": m_rt,
                            "gate_up_TFLOPs": e_gu["achieved"], "down_TFLOPs": e_d["achieved"], "router_projection_TFLOPs": e_r["achieved"],
                            "frac_of_mfma_peak": {"gate_up": e_gu["frac"], "down": e_d["frac"], "router_projection": e_r["frac"]},

@@ -124,8 +124,13 @@ OMNI_API int32_t omni_schedule_noalloc(const int32_t* indices, int32_t* offsets,
  *               of partial dot products (H*sizeof(elem)/8 must be 64..1024 bytes, a power of two; wider rows are
  *               taken in up to 64 column blocks of that form, one pair of launches per block, [8 * blocks][T][k] floats).
  *               Rows beyond 8 KiB exist for SPLIT only, and AUTO is SPLIT for them.
- *               AUTO = SPLIT when the tables overflow one L2 but an eighth of them fits and there
- *               are >= 32768 pairs (and for rows beyond 8 KiB), else GATHER.  SEGMENT is the expert-centric organisation:
+ *               AUTO chooses between GATHER and SPLIT from a measured grid, by the length of the row slice
+ *               each lane group streams (H*sizeof(elem)/8), the bytes of both tables and the pair count
+ *               T*k: GATHER below 32768 pairs, for tables of at most 3 MiB, for slices under 128 bytes
+ *               and for k > 128; SPLIT for 128-byte slices up to 32 MiB of tables from 131072 pairs, for
+ *               256-byte slices up to 128 MiB (from 65536 pairs, or from 16 MiB of tables), for longer
+ *               slices up to 256 MiB of tables or from 262144 pairs (and 2k >= lanes per row), and for
+ *               rows beyond 8 KiB.  SEGMENT is the expert-centric organisation:
  *               omni_schedule, a pass over the sorted pairs for the coefficients, a token pass
  *               for the sum; kept so that the organisations can be measured side by side.
  *               GATHER and SEGMENT agree bit for bit, SPLIT to fp32 rounding of the dot products.
@@ -327,9 +332,10 @@ OMNI_API int32_t omni_moe_fwd(const void* x, const void* gate_weight, const void
 
 /* omni_moe_fwd with the expert algorithm named by the caller (OMNI_EXPERT_ALGO_*; omni_moe_fwd is this call with
  * OMNI_EXPERT_ALGO_AUTO).  AUTO decides from sizes alone, without a device-to-host read; which algorithm is faster
- * also depends on how many DISTINCT experts the router picks, which only the caller can know: with tables far beyond
- * the caches but a skewed router (benchmark config 5: 2 GiB of tables, ~3700 live experts) SPLIT serves the live
- * rows from the XCDs' L2s where AUTO's GATHER fetches them over the fabric.  An algorithm that does not cover the
+ * also depends on how many DISTINCT experts the router picks, which only the caller can know: AUTO's rule is fitted
+ * to ids spread evenly over the tables, and a router that concentrates on few experts moves the crossover (what is
+ * live then fits the caches whatever the table size), so a caller who knows the skew may name the algorithm.
+ * An algorithm that does not cover the
  * shape is OMNI_ERR_UNSUPPORTED before anything is enqueued.  The workspace size depends on the algorithm.
  * No counterpart in the reference (its scheduler reads the id statistics back to the host, omni_scheduler.py:82,90). */
 OMNI_API size_t omni_moe_workspace_bytes_algo(int64_t num_tokens, int32_t hidden_size, int32_t intermediate_size,

@@ -549,9 +549,19 @@ static int expert_dense_dispatch(const void* x, const void* up, const void* down
   return omni_linear_fwd(coef, vt2, nullptr, y, T, (int32_t)(2 * N), H, dtype, s);
 }
 
-// What OMNI_EXPERT_ALGO_AUTO runs.  The split algorithm pays when the two tables overflow one
-// XCD's 4 MiB L2 while an eighth of them fits beside the streaming x and y rows, and when there
-// are enough pairs to amortise its second launch; otherwise rows are gathered whole.
+// What OMNI_EXPERT_ALGO_AUTO runs, from the sizes alone.  The split algorithm gives every XCD an eighth of each table row,
+// so it pays while an XCD's share of the tables stays near its caches (its 4 MiB L2 and its part of the memory-side cache)
+// and a row slice is long enough to fetch well; whole-row gathering wins on short rows, on tables far beyond the caches
+// and with few pairs (the split algorithm's second launch: at 32768 pairs it wins from 512-byte slices on, or from 16 MiB
+// of tables on with 256-byte slices).  Measured with ids uniform over the experts, bf16, 4096 /
+// 16384 / 32768 tokens x 16 / 16 / 32 experts per token, time of split over time of gather:
+//   slice  64 B (hidden  256): 1.3-3.4 at every table size                        -> gather
+//   slice 128 B (hidden  512): 0.72-0.91 up to 32 MiB of tables from 262144 pairs on, 1.02-1.6 beyond
+//   slice 256 B (hidden 1024): 0.49-0.67 up to 64 MiB, 0.95-1.01 at 256 MiB, 1.03-1.14 beyond
+//   slice 512 B (hidden 2048): 0.37-0.77 up to 128 MiB, 0.9 at 256 MiB; beyond, 0.89-0.99 from 262144 pairs on and 1.04-1.16 with 65536
+//   slice   1 KiB (hidden 4096): 0.59-0.95 with 32 experts per token (a token's pairs fill half of the 64 lanes that
+//                                share out a batch), 1.05-1.38 with 16
+// A skewed router (few live experts) moves every figure towards the split algorithm; the caller who knows says so.
 static int resolve_algo(int algo, int64_t T, int H, int64_t N, int k, int dtype) {
   if (algo != OMNI_EXPERT_ALGO_AUTO) return algo;
   // The dense algorithm is never chosen here: it multiplies every token by every table row, so one non-finite value
@@ -561,10 +571,14 @@ static int resolve_algo(int algo, int64_t T, int H, int64_t N, int k, int dtype)
   const int es = dtype == OMNI_F32 ? 4 : 2;
   // rows beyond 8 KiB do not fit the gather kernel's registers: the split kernels take them in column blocks
   if ((int64_t)H * es > 8192) return OMNI_EXPERT_ALGO_SPLIT;
-  const int64_t tables = 2 * N * (int64_t)H * es;
-  const bool fits = split_lanes_per_row(H, es) != 0 && k <= 2 * kWave;
-  if (fits && tables > (3ll << 20) && tables / kSlices <= (3ll << 20) && T * (int64_t)k >= 32768) return OMNI_EXPERT_ALGO_SPLIT;
-  return OMNI_EXPERT_ALGO_GATHER;
+  const int64_t tables = 2 * N * (int64_t)H * es, pairs = T * (int64_t)k;
+  const int lpr = split_lanes_per_row(H, es);           // 16-byte lanes per row slice: 4 .. 64, or 0
+  if (lpr < 8 || k > 2 * kWave || tables <= (3ll << 20) || pairs < 32768) return OMNI_EXPERT_ALGO_GATHER;
+  bool split;
+  if (lpr == 8) split = tables <= (32ll << 20) && pairs >= 131072;
+  else if (lpr == 16) split = tables <= (128ll << 20) && (pairs >= 65536 || tables >= (16ll << 20));
+  else split = (tables <= (256ll << 20) || pairs >= 262144) && 2 * k >= lpr;
+  return split ? OMNI_EXPERT_ALGO_SPLIT : OMNI_EXPERT_ALGO_GATHER;
 }
 
 // OMNI_OK when omni_expert_fwd takes `algo` for these sizes (what the whole-layer call checks before it enqueues anything).

@@ -104,8 +104,9 @@ class OmniMoE(nn.Module):
     # against 241, 16384 tokens 425-440 against 415, 65536 tokens 1.66-1.70 against 1.63 ms; benchmark config 5: 3.43 against 3.17 ms).
     overlap_max_work = 2 ** 36
     # Expert algorithm of the fused forward: "auto" decides from the sizes alone (no device-to-host read).  Which one is
-    # faster also depends on how many DISTINCT experts the router picks: with tables far beyond the caches and a skewed
-    # router (few live experts) "split" beats auto's "gather"; the caller who knows the distribution says so here.
+    # faster also depends on how many DISTINCT experts the router picks: auto's rule is fitted to ids spread evenly
+    # over the tables, and a router that concentrates on few experts moves the crossover between "gather" and "split";
+    # the caller who knows the distribution says so here.
     expert_algo = "auto"
 
     @staticmethod

@@ -286,12 +286,12 @@ def test_layer_config5_large_skewed(device):
 @pytest.mark.parametrize("two_streams", [False, True], ids=["one-stream", "two-streams"])
 def test_layer_expert_term_visible_auto_split(two_streams, dtype, training, device):
     """A layer whose expert branch is as large as its MLP branch (weights ~ N(0, 0.1)) and whose shape makes the layer call
-    pick the hidden-split expert algorithm (4096 tokens x 8 = 32768 pairs, tables that overflow one L2): y - mlp must equal
+    pick the hidden-split expert algorithm (4096 tokens x 32 = 131072 pairs, tables that overflow one L2): y - mlp must equal
     the oracle's expert term on the expert term's own scale, on one stream and on two.  A layer that dropped or mis-wired
     router -> experts (wrong gates or ids buffer, workspace overlap, missing join) fails here.  In training mode the router
     normalises with the statistics of the whole 4096-token batch, on the device and in the oracle."""
     from omni_moe.modules.omni_moe import OmniMoE, OmniMoEConfig
-    T, H, I, N, k = 4096, 512, 512, (1024 if dtype == torch.float32 else 4096), 8
+    T, H, I, N, k = 4096, 512, 512, (1024 if dtype == torch.float32 else 4096), 32
     x, w = oracle.make_layer_inputs(21, T, H, I, N, dtype=dtype, w_std=0.1)
     # the shared MLP scaled down to the size of the expert term (batch statistics flatten the gates: smaller still in training)
     w.down_proj = (w.down_proj.float() * (0.006 if training else 0.03)).to(dtype)

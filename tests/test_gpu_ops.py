@@ -131,8 +131,9 @@ EXPERT_CASES = [
     # (T, H, N, k, dtype, kind)
     (1024, 1024, 1024, 32, torch.bfloat16, "ref"),      # reference benchmark grid (tests/test_expert.py:181-187)
     (1024, 1024, 4096, 32, torch.bfloat16, "ref"),
-    (1024, 1024, 16384, 32, torch.bfloat16, "ref"),     #   ... its two larger tables: 64 MiB and 256 MiB, where AUTO
-    (1024, 1024, 65536, 32, torch.bfloat16, "ref"),     #   goes back from the hidden-split to the gather algorithm
+    (1024, 1024, 16384, 32, torch.bfloat16, "ref"),     #   ... its two larger tables: 64 MiB and 256 MiB
+    (1024, 1024, 65536, 32, torch.bfloat16, "ref"),
+    (4096, 1024, 16384, 16, torch.bfloat16, "ref"),     # 65536 pairs, 64 MiB of tables: AUTO takes the hidden-split algorithm
     (2048, 1024, 4096, 16, torch.bfloat16, "baseline"), # benchmark config 3 shape (token subset)
     (512, 256, 1024, 8, torch.float32, "baseline"),     # benchmark config 1 shape
     (256, 2048, 8192, 32, torch.bfloat16, "baseline"),  # benchmark config 5 row length
