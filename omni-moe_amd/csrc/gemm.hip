@@ -715,7 +715,10 @@ __device__ __forceinline__ void stream_epilogue(const GemmArgs& g, f32x4_t (&acc
       const auto s0 = __builtin_amdgcn_permlane16_swap(w[0][0], w[1][0], false, false);
       const auto s1 = __builtin_amdgcn_permlane16_swap(w[0][1], w[1][1], false, false);
       const int n = nb + (j + (g4 & 1)) * 16 + (g4 & 2) * 4;
-      if (m < g.M) *(u32x4_t*)(g.c + ((int64_t)m * g.N + n) * 2) = u32x4_t{s0[0], s1[0], s0[1], s1[1]};
+      if (m < g.M) {
+        if constexpr (EPI == kEpiSwiglu) __builtin_nontemporal_store(u32x4_t{s0[0], s1[0], s0[1], s1[1]}, (u32x4_t*)(g.c + ((int64_t)m * g.N + n) * 2));
+        else *(u32x4_t*)(g.c + ((int64_t)m * g.N + n) * 2) = u32x4_t{s0[0], s1[0], s0[1], s1[1]};
+      }
       if constexpr (EPI == kEpiSwiglu) {
         if (g.save_gate) {                               // the two rounded projections leave the same way (kept for a backward pass)
           uint32_t a[2][2], b[2][2];
@@ -829,6 +832,7 @@ __global__ __launch_bounds__(512, 1) void gemm_stream_kernel(const GemmArgs g) {
   clear_acc();
 
   int c_stage = 0;                                     // stage of the K tile being multiplied
+  constexpr int kEpiStores = (EPI == kEpiSwiglu) ? 8 : 16;   // store instructions of a wave's epilogue (no memory instruction follows them)
   // One K step of 32: TM*TN matrix instructions in row order, at most one memory instruction behind each (slot_op).
   // In the K tile's second step, whose following step reads the other stage, the wave waits after row 0 for its fragment
   // reads and ring loads and meets the block.
@@ -838,11 +842,15 @@ __global__ __launch_bounds__(512, 1) void gemm_stream_kernel(const GemmArgs g) {
   auto slot_op = [](bool second, int i, int j) constexpr -> int {
     if (j == 0 && i >= 1 && i <= 4) return 10 + (i - 1);
     if (j == 1 && i >= 1 && i <= 4) return second ? 30 + (i - 1) : 34 + (i - 1);
+    if (second && j == 1 && i >= 5) return 40 + (i - 5);            // 40-43: the weight rows too, in a tile's last K tile
+    if (second && j == 2 && i == 7) return 43;
     if (j == 2 && i == 1) return 20;
     if (j == 3 && i >= 1) return 20 + i;
     return 0;
   };
-  auto kstep = [&](auto ks_tag, auto sync_tag) __attribute__((always_inline)) {
+  // last: the output tile's last K tile; young: memory instructions of the wave issued after the loads this K tile's sync
+  // point waits for (the previous tile's stores, when the K tile is a tile's first)
+  auto kstep = [&](auto ks_tag, auto sync_tag, const bool last, const int young) __attribute__((always_inline)) {
     constexpr int ks = decltype(ks_tag)::value;
     constexpr bool sync = decltype(sync_tag)::value;
     constexpr int nks = ks ^ 1;
@@ -858,13 +866,17 @@ __global__ __launch_bounds__(512, 1) void gemm_stream_kernel(const GemmArgs g) {
         if (op >= 10 && op < 20) read_b(rs, nks, op - 10);
         if (op >= 20 && op < 30) read_a(rs, nks, op - 20);
         if (op >= 30 && op < 34) { if (fa) issue_one(op - 30); }
-        if (op >= 34) { if (half_pending) issue_one(op - 30); }
+        if (op >= 34 && op < 40) { if (half_pending) issue_one(op - 30); }
+        if (op >= 40) { if (fa && last) issue_one(op - 36); }
         __builtin_amdgcn_sched_barrier(0);
       }
       if constexpr (sync) {
         if (i == kSyncRow) {
           wait_lds_reads();                            // this wave holds every fragment of the K tile
-          wait_vmcnt<0>();                             // the next K tile has landed
+          // the next K tile has landed.  The counter runs in issue order, loads and stores alike: behind a tile's epilogue
+          // its stores are younger than every load of the next K tile (whose weight rows a tile's last K tile requests
+          // early for that reason) and may stay in flight for another K tile
+          if (young == kEpiStores) wait_vmcnt<kEpiStores>(); else wait_vmcnt<0>();
           __builtin_amdgcn_s_barrier();                // ... for all waves; this K tile's stage is free
           __builtin_amdgcn_sched_barrier(0);
         }
@@ -872,12 +884,13 @@ __global__ __launch_bounds__(512, 1) void gemm_stream_kernel(const GemmArgs g) {
     }
   };
   using I0 = std::integral_constant<int, 0>; using I1 = std::integral_constant<int, 1>;
-  auto k_tile = [&]() __attribute__((always_inline)) {
-    kstep(I0{}, std::false_type{});                    // the weights of the K tile whose activations were requested one step ago
+  auto k_tile = [&](const bool last, const int young) __attribute__((always_inline)) {
+    kstep(I0{}, std::false_type{}, last, 0);           // the weights of the K tile whose activations were requested one step ago
     if (half_pending) { cursor_advance(); half_pending = false; }
     const bool fa = f_tile < num_tiles;
-    kstep(I1{}, std::true_type{});                     // the activations of the K tile two ahead go into the freed stage
-    half_pending = fa;
+    kstep(I1{}, std::true_type{}, last, young);        // the activations of the K tile two ahead go into the freed stage
+    if (last && fa) cursor_advance();                  // ... with its weights, when the epilogue comes next
+    half_pending = fa && !last;
     c_stage ^= 1;
   };
 
@@ -895,11 +908,14 @@ __global__ __launch_bounds__(512, 1) void gemm_stream_kernel(const GemmArgs g) {
 #pragma unroll
   for (int j = 0; j < TN; ++j) read_b(0, 0, j);
 
+  int young = 0;                                       // stores of the previous tile's epilogue, if their number is known
   for (int tile = blockIdx.x; tile < num_tiles; tile += gridDim.x) {
-    for (int kt = 0; kt < num_kt; ++kt) k_tile();
+    for (int kt = 0; kt < num_kt; ++kt) k_tile(kt == num_kt - 1, kt == 0 ? young : 0);
     int tm, tn;
     tile_coords_of(g, tile, tm, tn);
     stream_epilogue<DT, EPI>(g, acc, tm * BM, tn * BN, wm, wn, lane);
+    // every row of the wave inside the matrix: each store instruction of the epilogue has been issued
+    young = (g.M - tm * BM - wm * 128 >= 128 && !(EPI == kEpiSwiglu && g.save_gate)) ? kEpiStores : 0;
     clear_acc();
   }
 }
