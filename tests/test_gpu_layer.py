@@ -22,7 +22,8 @@ def _ops():
 
 # the first four are the reference's benchmark grid (tests/test_mlp.py:144-150): intermediate 1024 .. 65536
 MLP_CASES = [(1024, 1024, 1024), (1024, 1024, 4096), (1024, 1024, 16384), (1024, 1024, 65536), (4096, 1024, 4096), (4100, 1024, 4096),
-             (333, 256, 1000), (128, 64, 128), (512, 2048, 8192), (5, 8, 8)]
+             (333, 256, 1000), (128, 64, 128), (512, 2048, 8192), (5, 8, 8),
+             (8192, 128, 4096), (8200, 192, 2048)]      # streaming gate/up kernel with two and three K tiles per output tile, four tiles per block
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
