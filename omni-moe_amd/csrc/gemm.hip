@@ -715,10 +715,7 @@ __device__ __forceinline__ void stream_epilogue(const GemmArgs& g, f32x4_t (&acc
       const auto s0 = __builtin_amdgcn_permlane16_swap(w[0][0], w[1][0], false, false);
       const auto s1 = __builtin_amdgcn_permlane16_swap(w[0][1], w[1][1], false, false);
       const int n = nb + (j + (g4 & 1)) * 16 + (g4 & 2) * 4;
-      if (m < g.M) {
-        if constexpr (EPI == kEpiSwiglu) __builtin_nontemporal_store(u32x4_t{s0[0], s1[0], s0[1], s1[1]}, (u32x4_t*)(g.c + ((int64_t)m * g.N + n) * 2));
-        else *(u32x4_t*)(g.c + ((int64_t)m * g.N + n) * 2) = u32x4_t{s0[0], s1[0], s0[1], s1[1]};
-      }
+      if (m < g.M) *(u32x4_t*)(g.c + ((int64_t)m * g.N + n) * 2) = u32x4_t{s0[0], s1[0], s0[1], s1[1]};
       if constexpr (EPI == kEpiSwiglu) {
         if (g.save_gate) {                               // the two rounded projections leave the same way (kept for a backward pass)
           uint32_t a[2][2], b[2][2];
@@ -910,6 +907,10 @@ __global__ __launch_bounds__(512, 1) void gemm_stream_kernel(const GemmArgs g) {
 
   int young = 0;                                       // stores of the previous tile's epilogue, if their number is known
   for (int tile = blockIdx.x; tile < num_tiles; tile += gridDim.x) {
+    // (not unrolled, which would include peeling the first K tile off as a second loop body: the compiler then gives the
+    // accumulators different registers in the two bodies and the kernel needs 250 VGPRs instead of 216, which leaves no
+    // room on a SIMD for a wave of the kernels that the layer runs beside this one)
+#pragma clang loop unroll(disable)
     for (int kt = 0; kt < num_kt; ++kt) k_tile(kt == num_kt - 1, kt == 0 ? young : 0);
     int tm, tn;
     tile_coords_of(g, tile, tm, tn);
