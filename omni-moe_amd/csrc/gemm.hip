@@ -670,16 +670,37 @@ __device__ __forceinline__ f32x4_t mfma16(const u32x4_t a, const u32x4_t b, f32x
 
 // Epilogue of the streaming kernel (full column tiles, 16-byte stores; rows past M are not stored).  Lanes l and l ^ 16 hold columns 4g..4g+3 and 4g+4..4g+7 of
 // two neighbouring column tiles: one v_permlane16_swap per word leaves every lane with 8 consecutive columns of one
-// of the two tiles, so each store instruction writes 64 consecutive bytes of 16 rows.
+// of the two tiles, 64 consecutive bytes of a row over the four lanes l, l + 16, l + 32, l + 48.  The store path wants
+// those four in CONSECUTIVE lanes: a store-only microbenchmark moves 14 bytes per cycle and CU when neighbouring lanes
+// write different rows (16 rows x 64 bytes or 8 rows x 128 bytes per instruction alike) and 26-27 when each quad of
+// lanes writes 64 bytes on end, in any order of its four pieces; and while a tile's stores pass through that path the
+// ring loads of the next tile queue behind them.  So every word goes through one ds_bpermute_b32 (lane d takes from
+// lane d / 4 + 16 (d % 4); no LDS memory involved), after which lane d holds 16 bytes of row d / 4.  The residual is
+// fetched in that layout as well, 16 bytes per lane, and added to the rounded product there: the same arithmetic.
+__device__ __forceinline__ u32x4_t to_row_quads(const uint32_t x0, const uint32_t x1, const uint32_t x2, const uint32_t x3, const int from) {
+  return u32x4_t{(uint32_t)__builtin_amdgcn_ds_bpermute(from, (int)x0), (uint32_t)__builtin_amdgcn_ds_bpermute(from, (int)x1),
+                 (uint32_t)__builtin_amdgcn_ds_bpermute(from, (int)x2), (uint32_t)__builtin_amdgcn_ds_bpermute(from, (int)x3)};
+}
+template <int DT> __device__ __forceinline__ float half_lo(const uint32_t w) {
+  if constexpr (DT == kBF16) return bf16_lo(w); else return f16_bits_to_f32((uint16_t)(w & 0xffffu));
+}
+template <int DT> __device__ __forceinline__ float half_hi(const uint32_t w) {
+  if constexpr (DT == kBF16) return bf16_hi(w); else return f16_bits_to_f32((uint16_t)(w >> 16));
+}
 template <int DT, int EPI>
 __device__ __forceinline__ void stream_epilogue(const GemmArgs& g, f32x4_t (&acc)[8][4], const int m0, const int n0, const int wm,
                                                   const int wn, const int lane) {
   constexpr int TNO = (EPI == kEpiSwiglu) ? 2 : 4;
-  const int g4 = lane >> 4;
   const int nb = n0 + wn * (TNO * 16);
+  // (not for the SwiGLU form, whose epilogue is bound by its arithmetic: there the exchange costs the layer step 0.4 %)
+  constexpr bool kQuads = EPI != kEpiSwiglu;
+  const int tr = kQuads ? lane >> 2 : lane & 15;       // where the lane's 16 bytes go: row of the 16,
+  const int tg = kQuads ? lane & 3 : lane >> 4;        // ... piece of the row's 64 bytes
+  const int from = (tr + 16 * tg) * 4;                 // ds_bpermute address of the lane that holds them before the exchange
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
-    const int m = m0 + wm * 128 + i * 16 + (lane & 15);
+    const int m = m0 + wm * 128 + i * 16 + tr;
+    const bool stored = m < g.M;
 #pragma unroll
     for (int j = 0; j < TNO; j += 2) {
       uint32_t w[2][2];
@@ -696,26 +717,25 @@ __device__ __forceinline__ void stream_epilogue(const GemmArgs& g, f32x4_t (&acc
             v[q] = acc[i][j + t][q];
           }
         }
-        if constexpr (EPI == kEpiResidual) {
-          const int mr = m < g.M ? m : g.M - 1;          // rows past the matrix are exchanged but never stored
-          const u32x2_t r = *(const u32x2_t*)(g.res + ((int64_t)mr * g.N + nb + (j + t) * 16 + g4 * 4) * 2);
-          const uint32_t r0 = r[0], r1 = r[1];
-          if constexpr (DT == kBF16) {
-            v[0] = Elem<DT>::round(v[0]) + bf16_lo(r0); v[1] = Elem<DT>::round(v[1]) + bf16_hi(r0);
-            v[2] = Elem<DT>::round(v[2]) + bf16_lo(r1); v[3] = Elem<DT>::round(v[3]) + bf16_hi(r1);
-          } else {
-            v[0] = Elem<DT>::round(v[0]) + f16_bits_to_f32(r0 & 0xffff); v[1] = Elem<DT>::round(v[1]) + f16_bits_to_f32(r0 >> 16);
-            v[2] = Elem<DT>::round(v[2]) + f16_bits_to_f32(r1 & 0xffff); v[3] = Elem<DT>::round(v[3]) + f16_bits_to_f32(r1 >> 16);
-          }
-        }
         w[t][0] = pack2<DT>(v[0], v[1]);
         w[t][1] = pack2<DT>(v[2], v[3]);
       }
       // odd 16-lane rows of tile j's words change places with even rows of tile j+1's
       const auto s0 = __builtin_amdgcn_permlane16_swap(w[0][0], w[1][0], false, false);
       const auto s1 = __builtin_amdgcn_permlane16_swap(w[0][1], w[1][1], false, false);
-      const int n = nb + (j + (g4 & 1)) * 16 + (g4 & 2) * 4;
-      if (m < g.M) *(u32x4_t*)(g.c + ((int64_t)m * g.N + n) * 2) = u32x4_t{s0[0], s1[0], s0[1], s1[1]};
+      u32x4_t out = kQuads ? to_row_quads(s0[0], s1[0], s0[1], s1[1], from) : u32x4_t{s0[0], s1[0], s0[1], s1[1]};
+      const int n = nb + (j + (tg & 1)) * 16 + (tg & 2) * 4;
+      const int64_t at = ((int64_t)m * g.N + n) * 2;
+      if constexpr (EPI == kEpiResidual) {
+        const int mr = stored ? m : g.M - 1;             // rows past the matrix are computed but never stored
+        const u32x4_t r = *(const u32x4_t*)(g.res + ((int64_t)mr * g.N + n) * 2);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const uint32_t o = out[q], rq = r[q];
+          out[q] = pack2<DT>(half_lo<DT>(o) + half_lo<DT>(rq), half_hi<DT>(o) + half_hi<DT>(rq));
+        }
+      }
+      if (stored) *(u32x4_t*)(g.c + at) = out;
       if constexpr (EPI == kEpiSwiglu) {
         if (g.save_gate) {                               // the two rounded projections leave the same way (kept for a backward pass)
           uint32_t a[2][2], b[2][2];
@@ -730,9 +750,10 @@ __device__ __forceinline__ void stream_epilogue(const GemmArgs& g, f32x4_t (&acc
           const auto a1 = __builtin_amdgcn_permlane16_swap(a[0][1], a[1][1], false, false);
           const auto b0 = __builtin_amdgcn_permlane16_swap(b[0][0], b[1][0], false, false);
           const auto b1 = __builtin_amdgcn_permlane16_swap(b[0][1], b[1][1], false, false);
-          if (m < g.M) {
-            *(u32x4_t*)(g.save_gate + ((int64_t)m * g.N + n) * 2) = u32x4_t{a0[0], a1[0], a0[1], a1[1]};
-            *(u32x4_t*)(g.save_up + ((int64_t)m * g.N + n) * 2) = u32x4_t{b0[0], b1[0], b0[1], b1[1]};
+          const u32x4_t ga = {a0[0], a1[0], a0[1], a1[1]}, ub = {b0[0], b1[0], b0[1], b1[1]};
+          if (stored) {
+            *(u32x4_t*)(g.save_gate + at) = ga;
+            *(u32x4_t*)(g.save_up + at) = ub;
           }
         }
       }
