@@ -790,53 +790,70 @@ __global__ __launch_bounds__(512, 1) void gemm_stream_kernel(const GemmArgs g) {
   const uint32_t b_voff = (uint32_t)((EPI == kEpiSwiglu ? (wave & 3) * 8 : wave * 8) + (lane >> 3)) * row_bytes + sw * 16;
   constexpr int kBRowsPerInstr = (EPI == kEpiSwiglu) ? 32 : 64;     // weight rows between consecutive load instructions of a wave
 
-  // fetch cursor: the next K tile of the stream to request
-  int f_tile = blockIdx.x, f_kt = 0, f_stage = 0;
-  bool half_pending = false;                          // the cursor's K tile has its activation half requested, not yet its weights
-  uint32_t f_a = 0, f_b = 0;                          // byte offsets of the tile's first activation / weight row
-  bool f_hi = false;                                  // ... the weight row counted in the second weight matrix
-  auto cursor_coords = [&]() {
+  uint32_t b_voff4[4];                                 // ... and per weight load instruction of the wave
+#pragma unroll
+  for (int q = 0; q < 4; ++q) b_voff4[q] = b_voff + (uint32_t)(q * kBRowsPerInstr) * row_bytes;
+
+  // Fetch cursor: the next K tile of the stream to request.  Everything a load instruction needs beyond its lane offsets is
+  // kept ready in scalar registers and moved on once per K tile (the K loop otherwise spends four scalar instructions
+  // on every matrix instruction, and a wave issues in order): the LDS address of the wave's first row in the cursor's
+  // stage, the byte offset of the K tile within the activation and the weight rows, the weight matrix's descriptor.
+  using LdsPtr = __attribute__((address_space(3))) void*;
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(LdsPtr)lds;
+  int f_tile = blockIdx.x, f_kt = 0;
+  uint32_t f_ldsw = lds_base + (uint32_t)wave * 1024;  // ... of the wave's first row in the cursor's stage
+  int f_flip = kStage;                                 // to the other stage and back
+  uint32_t f_sa = 0, f_sb = 0;
+  int half_pending = 0;                                // the cursor's K tile has its activation half requested, not yet its weights (an int: a bool carried round the loop becomes a lane mask)
+  __amdgpu_buffer_rsrc_t rsrc_w = rsrc_b;              // the second weight matrix for the upper half of the columns (plain and residual forms)
+  auto cursor_coords = [&]() {                         // at a tile's first K tile
     int tm, tn;
     tile_coords_of(g, f_tile, tm, tn);
-    f_a = (uint32_t)(tm * BM) * row_bytes;
-    f_hi = EPI != kEpiSwiglu && g.b1 != nullptr && tn * BN >= g.N / 2;
-    f_b = (uint32_t)(tn * BN - (f_hi ? g.N / 2 : 0)) * row_bytes;
+    f_sa = (uint32_t)(tm * BM) * row_bytes;
+    const bool hi = EPI != kEpiSwiglu && g.b1 != nullptr && tn * BN >= g.N / 2;
+    rsrc_w = hi ? rsrc_hi : rsrc_b;
+    f_sb = (uint32_t)(tn * BN - (hi ? g.N / 2 : 0)) * row_bytes;
     const int last = g.M - 1 - tm * BM;                // last row of the matrix, counted from the tile's first: a ragged last tile re-reads it
 #pragma unroll
     for (int q = 0; q < 4; ++q) a_voff[q] = (uint32_t)min(q * 64 + wave * 8 + (lane >> 3), last) * row_bytes + sw * 16;
   };
   cursor_coords();
   auto issue_one = [&](int q) __attribute__((always_inline)) {       // q = 0..3: activation rows, 4..7: weight rows
-    uint8_t* st = lds + f_stage * kStage;
     if (q < 4)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (__attribute__((address_space(3))) void*)(st + (8 * q + wave) * 1024), 16, a_voff[q],
-                                               f_a + f_kt * 128, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (LdsPtr)(uintptr_t)(f_ldsw + q * 8192), 16, a_voff[q], f_sa, 0, 0);
     else
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(f_hi ? rsrc_hi : rsrc_b, (__attribute__((address_space(3))) void*)(st + BM * kRow + (8 * (q - 4) + wave) * 1024),
-                                               16, b_voff, f_b + (uint32_t)((q - 4) * kBRowsPerInstr) * row_bytes + f_kt * 128, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_w, (LdsPtr)(uintptr_t)(f_ldsw + BM * kRow + (q - 4) * 8192), 16, b_voff4[q - 4], f_sb, 0, 0);
   };
   auto cursor_advance = [&]() {                        // after a K tile's second half has been issued
-    f_stage ^= 1;
+    f_ldsw += (uint32_t)f_flip;
+    f_flip = -f_flip;
     if (++f_kt == num_kt) {
       f_kt = 0;
       f_tile += gridDim.x;
       if (f_tile < num_tiles) cursor_coords();
+    } else {
+      f_sa += 128;
+      f_sb += 128;
     }
   };
 
-  // fragment reads: lane reads row lane%16 of a 16-row tile, logical chunk 4*kstep + lane/16 (8 K values of the step's 32)
+  // fragment reads: lane reads row lane%16 of a 16-row tile, logical chunk 4*kstep + lane/16 (8 K values of the step's 32).
+  // ra[1], rb[1]: the lane's activation / weight fragment row of K step 1 in the stage being multiplied; ra[0], rb[0]: of K step 0
+  // in the OTHER stage (the next K tile's) -- what the first and the second step of a K tile read for the step after them;
+  // the row tile comes as the instruction's immediate offset, and the four change stages once per K tile (c_flip).
   const int r16 = lane & 15;
-  int off_ks[2];
+  uint32_t ra[2], rb[2];
 #pragma unroll
-  for (int ks = 0; ks < 2; ++ks) off_ks[ks] = r16 * kRow + ((4 * ks + (lane >> 4)) ^ (r16 >> 1)) * 16;
-  const int a_frag = (wm * 128) * kRow, b_frag = BM * kRow + (wn * 64) * kRow;
+  for (int ks = 0; ks < 2; ++ks) {
+    const uint32_t off = lds_base + (uint32_t)(r16 * kRow + ((4 * ks + (lane >> 4)) ^ (r16 >> 1)) * 16) + (ks == 0 ? (uint32_t)kStage : 0u);
+    ra[ks] = (uint32_t)((wm * 128) * kRow) + off;
+    rb[ks] = (uint32_t)(BM * kRow + (wn * 64) * kRow) + off;
+  }
+  int c_flip[2] = {-kStage, kStage};                   // next change of ra[ks], rb[ks]
+  using LdsFrag = const __attribute__((address_space(3))) u32x4_t*;
   u32x4_t af[TM], bf[2][TN];
-  auto read_a = [&](int stage, int ks, int i) __attribute__((always_inline)) {
-    af[i] = *(const u32x4_t*)(lds + stage * kStage + a_frag + i * 16 * kRow + off_ks[ks]);
-  };
-  auto read_b = [&](int stage, int ks, int j) __attribute__((always_inline)) {
-    bf[ks][j] = *(const u32x4_t*)(lds + stage * kStage + b_frag + j * 16 * kRow + off_ks[ks]);
-  };
+  auto read_a = [&](int ks, int i) __attribute__((always_inline)) { af[i] = *(LdsFrag)(uintptr_t)(ra[ks] + i * 16 * kRow); };
+  auto read_b = [&](int ks, int j) __attribute__((always_inline)) { bf[ks][j] = *(LdsFrag)(uintptr_t)(rb[ks] + j * 16 * kRow); };
 
   f32x4_t acc[TM][TN];
   auto clear_acc = [&]() __attribute__((always_inline)) {
@@ -849,7 +866,6 @@ __global__ __launch_bounds__(512, 1) void gemm_stream_kernel(const GemmArgs g) {
   };
   clear_acc();
 
-  int c_stage = 0;                                     // stage of the K tile being multiplied
   constexpr int kEpiStores = (EPI == kEpiSwiglu) ? 8 : 16;   // store instructions of a wave's epilogue (no memory instruction follows them)
   // One K step of 32: TM*TN matrix instructions in row order, at most one memory instruction behind each (slot_op).
   // In the K tile's second step, whose following step reads the other stage, the wave waits after row 0 for its fragment
@@ -868,12 +884,14 @@ __global__ __launch_bounds__(512, 1) void gemm_stream_kernel(const GemmArgs g) {
   };
   // last: the output tile's last K tile; young: memory instructions of the wave issued after the loads this K tile's sync
   // point waits for (the previous tile's stores, when the K tile is a tile's first)
-  auto kstep = [&](auto ks_tag, auto sync_tag, const bool last, const int young) __attribute__((always_inline)) {
+  auto kstep = [&](auto ks_tag, auto sync_tag, const int last, const int young) __attribute__((always_inline)) {
     constexpr int ks = decltype(ks_tag)::value;
     constexpr bool sync = decltype(sync_tag)::value;
     constexpr int nks = ks ^ 1;
-    const int rs = sync ? c_stage ^ 1 : c_stage;      // stage the following step's fragments come from
-    const bool fa = f_tile < num_tiles;                // the cursor's K tile exists
+    // (scalar registers by force: left alone the compiler keeps these loop-carried flags in vector registers and tests them there)
+    const bool fa = f_tile < num_tiles;
+    const bool hp = half_pending != 0;
+    const bool fl = fa && last;
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
 #pragma unroll
@@ -881,11 +899,11 @@ __global__ __launch_bounds__(512, 1) void gemm_stream_kernel(const GemmArgs g) {
         acc[i][j] = mfma16<DT>(bf[ks][j], af[i], acc[i][j]);
         __builtin_amdgcn_sched_barrier(0);
         const int op = slot_op(sync, i, j);
-        if (op >= 10 && op < 20) read_b(rs, nks, op - 10);
-        if (op >= 20 && op < 30) read_a(rs, nks, op - 20);
+        if (op >= 10 && op < 20) read_b(nks, op - 10);
+        if (op >= 20 && op < 30) read_a(nks, op - 20);
         if (op >= 30 && op < 34) { if (fa) issue_one(op - 30); }
-        if (op >= 34 && op < 40) { if (half_pending) issue_one(op - 30); }
-        if (op >= 40) { if (fa && last) issue_one(op - 36); }
+        if (op >= 34 && op < 40) { if (hp) issue_one(op - 30); }
+        if (op >= 40) { if (fl) issue_one(op - 36); }
         __builtin_amdgcn_sched_barrier(0);
       }
       if constexpr (sync) {
@@ -902,14 +920,15 @@ __global__ __launch_bounds__(512, 1) void gemm_stream_kernel(const GemmArgs g) {
     }
   };
   using I0 = std::integral_constant<int, 0>; using I1 = std::integral_constant<int, 1>;
-  auto k_tile = [&](const bool last, const int young) __attribute__((always_inline)) {
+  auto k_tile = [&](const int last, const int young) __attribute__((always_inline)) {
     kstep(I0{}, std::false_type{}, last, 0);           // the weights of the K tile whose activations were requested one step ago
-    if (half_pending) { cursor_advance(); half_pending = false; }
-    const bool fa = f_tile < num_tiles;
+    if (half_pending) { cursor_advance(); half_pending = 0; }
+    const int fa = f_tile < num_tiles ? 1 : 0;
     kstep(I1{}, std::true_type{}, last, young);        // the activations of the K tile two ahead go into the freed stage
-    if (last && fa) cursor_advance();                  // ... with its weights, when the epilogue comes next
-    half_pending = fa && !last;
-    c_stage ^= 1;
+    if (last & fa) cursor_advance();                   // ... with its weights, when the epilogue comes next
+    half_pending = fa & (last ^ 1);
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) { ra[ks] += (uint32_t)c_flip[ks]; rb[ks] += (uint32_t)c_flip[ks]; c_flip[ks] = -c_flip[ks]; }
   };
 
   // ---- prologue: the stream's first two K tiles
@@ -922,9 +941,9 @@ __global__ __launch_bounds__(512, 1) void gemm_stream_kernel(const GemmArgs g) {
   wait_vmcnt<8>();                                     // the first K tile has landed
   __builtin_amdgcn_s_barrier();
 #pragma unroll
-  for (int i = 0; i < TM; ++i) read_a(0, 0, i);
+  for (int i = 0; i < TM; ++i) af[i] = *(LdsFrag)(uintptr_t)(ra[0] - (uint32_t)kStage + i * 16 * kRow);     // K step 0 of stage 0
 #pragma unroll
-  for (int j = 0; j < TN; ++j) read_b(0, 0, j);
+  for (int j = 0; j < TN; ++j) bf[0][j] = *(LdsFrag)(uintptr_t)(rb[0] - (uint32_t)kStage + j * 16 * kRow);
 
   int young = 0;                                       // stores of the previous tile's epilogue, if their number is known
   for (int tile = blockIdx.x; tile < num_tiles; tile += gridDim.x) {
@@ -932,7 +951,7 @@ __global__ __launch_bounds__(512, 1) void gemm_stream_kernel(const GemmArgs g) {
     // accumulators different registers in the two bodies and the kernel needs 250 VGPRs instead of 216, which leaves no
     // room on a SIMD for a wave of the kernels that the layer runs beside this one)
 #pragma clang loop unroll(disable)
-    for (int kt = 0; kt < num_kt; ++kt) k_tile(kt == num_kt - 1, kt == 0 ? young : 0);
+    for (int kt = 0; kt < num_kt; ++kt) k_tile(kt == num_kt - 1 ? 1 : 0, kt == 0 ? young : 0);
     int tm, tn;
     tile_coords_of(g, tile, tm, tn);
     stream_epilogue<DT, EPI>(g, acc, tm * BM, tn * BN, wm, wn, lane);
