@@ -309,10 +309,21 @@ __device__ __forceinline__ float reduce_scatter_group(float (&v)[N], const int l
 // A wave owns GP = 64 / LPR tokens, one per lane group; the group's LPR lanes cover the token's
 // row slice, 16 bytes each.  Pairs go in batches of LPR: LPR partial dot products per lane,
 // then one reduce-scatter leaves pair `sub` of the batch in lane `sub`.
-template <int DT, int LPR>
+// SMALL: every table, x, y and the partial sums stay below 4 GiB, ids and row lengths below 2^24 (split_offsets_small):
+// a row's byte offset is then one full-rate v_mad_u32_u24 on 32-bit lane offsets instead of a 64-bit multiply-add and two
+// 32-bit multiplies at a quarter of the rate -- address arithmetic was more than half of the vector instructions' time here.
+template <bool SMALL> struct SplitOff { using type = int64_t; };
+template <> struct SplitOff<true> { using type = uint32_t; };
+template <bool SMALL>
+__device__ __forceinline__ typename SplitOff<SMALL>::type split_mul(uint32_t a, typename SplitOff<SMALL>::type b) {
+  if constexpr (SMALL) return __umul24(a, b); else return (int64_t)a * b;
+}
+
+template <int DT, int LPR, bool SMALL>
 __global__ __launch_bounds__(kTokensPerBlock* kWave) void expert_split_dots_kernel(
     const uint8_t* __restrict__ x, const uint8_t* __restrict__ up, const int32_t* __restrict__ ids,
     float* __restrict__ partial, int num_tokens, int hidden, int top_k, uint32_t num_experts, int col_block) {
+  using Off = typename SplitOff<SMALL>::type;
   constexpr int E = Row16<DT>::kElems, GP = kWave / LPR;
   constexpr int LD = LPR < 8 ? LPR : 8;                          // row loads in flight at a time
   const int lane = lane_id(), sub = lane % LPR, grp = lane / LPR;
@@ -320,11 +331,11 @@ __global__ __launch_bounds__(kTokensPerBlock* kWave) void expert_split_dots_kern
   const int t = ((int)(blockIdx.x / kSlices) * kTokensPerBlock + (threadIdx.x >> 6)) * GP + grp;
   const bool live = t < num_tokens;
   const int tt = live ? t : 0;
-  const int64_t row_bytes = int64_t(hidden) * (16 / E);
+  const Off row_bytes = Off(hidden) * (16 / E);
   // this lane's 16 bytes inside a row (rows wider than 8 slices of 64 lanes go in column blocks of 8 slices, one launch each)
-  const int64_t col = (int64_t(col_block) * kSlices + slice) * LPR * 16 + sub * 16;
-  const u32x4_t xr = *(const u32x4_t*)(x + tt * row_bytes + col);
-  const int64_t base = int64_t(tt) * top_k;
+  const Off col = (Off(col_block) * kSlices + slice) * LPR * 16 + sub * 16;
+  const u32x4_t xr = *(const u32x4_t*)(x + (split_mul<SMALL>((uint32_t)tt, row_bytes) + col));
+  const Off base = split_mul<SMALL>((uint32_t)tt, (Off)top_k);
   for (int jb = 0; jb < top_k; jb += LPR) {
     // lane `sub` of a group fetches the id of pair `sub` of the batch; the group reads the ids from its lanes
     const int my_id = ids[base + min(jb + sub, top_k - 1)];
@@ -335,7 +346,7 @@ __global__ __launch_bounds__(kTokensPerBlock* kWave) void expert_split_dots_kern
 #pragma unroll
       for (int e = 0; e < LD; ++e) {
         const int id = __shfl(my_id, grp * LPR + e0 + e, kWave);
-        ur[e] = *(const u32x4_t*)(up + int64_t((uint32_t)id < num_experts ? id : 0) * row_bytes + col);
+        ur[e] = *(const u32x4_t*)(up + (split_mul<SMALL>((uint32_t)id < num_experts ? (uint32_t)id : 0u, row_bytes) + col));
       }
 #pragma unroll
       for (int e = 0; e < LD; ++e) d[e0 + e] = dot16<DT>(xr, ur[e], 0.f);
@@ -344,7 +355,7 @@ __global__ __launch_bounds__(kTokensPerBlock* kWave) void expert_split_dots_kern
     const int j = jb + sub;
     if (live && j < top_k) {
       const bool ok = (uint32_t)my_id < num_experts;
-      partial[((int64_t(col_block) * kSlices + slice) * num_tokens + t) * top_k + j] = ok ? total : 0.f;
+      partial[((Off(col_block) * kSlices + slice) * num_tokens + t) * top_k + j] = ok ? total : 0.f;
     }
   }
 }
@@ -354,11 +365,12 @@ __global__ __launch_bounds__(kTokensPerBlock* kWave) void expert_split_dots_kern
 // fetching its 16 bytes of the down row and the pair's coefficient from the lane that holds it.
 // WIDE: rows of several column blocks (col_block of col_blocks); otherwise both are compile-time constants, which keeps
 // the eight partial-sum loads of the common case one unrolled group that the compiler places behind the row requests.
-template <int DT, int LPR, bool WIDE>
+template <int DT, int LPR, bool WIDE, bool SMALL>
 __global__ __launch_bounds__(kTokensPerBlock* kWave) void expert_split_accumulate_kernel(
     const uint8_t* __restrict__ down, const void* __restrict__ gates, const int32_t* __restrict__ ids,
     const float* __restrict__ partial, uint8_t* __restrict__ y, int num_tokens, int hidden, int top_k, uint32_t num_experts,
     int col_block_arg, int col_blocks_arg) {
+  using Off = typename SplitOff<SMALL>::type;
   const int col_block = WIDE ? col_block_arg : 0, col_blocks = WIDE ? col_blocks_arg : 1;
   constexpr int E = Row16<DT>::kElems, GP = kWave / LPR;
   constexpr int LD = LPR < 8 ? LPR : 8;
@@ -367,9 +379,9 @@ __global__ __launch_bounds__(kTokensPerBlock* kWave) void expert_split_accumulat
   const int t = ((int)(blockIdx.x / kSlices) * kTokensPerBlock + (threadIdx.x >> 6)) * GP + grp;
   const bool live = t < num_tokens;
   const int tt = live ? t : 0;
-  const int64_t row_bytes = int64_t(hidden) * (16 / E);
-  const int64_t col = (int64_t(col_block) * kSlices + slice) * LPR * 16 + sub * 16;
-  const int64_t base = int64_t(tt) * top_k;
+  const Off row_bytes = Off(hidden) * (16 / E);
+  const Off col = (Off(col_block) * kSlices + slice) * LPR * 16 + sub * 16;
+  const Off base = split_mul<SMALL>((uint32_t)tt, (Off)top_k);
   float acc[E];
 #pragma unroll
   for (int i = 0; i < E; ++i) acc[i] = 0.f;
@@ -387,7 +399,7 @@ __global__ __launch_bounds__(kTokensPerBlock* kWave) void expert_split_accumulat
     auto request = [&](int slot, int e) {
       const int id = __shfl(my_id, grp * LPR + e, kWave);         // from the lane of this group that holds pair e
       used[slot] = id >= 0;
-      vr[slot] = *(const u32x4_t*)(down + int64_t(used[slot] ? id : 0) * row_bytes + col);
+      vr[slot] = *(const u32x4_t*)(down + (split_mul<SMALL>(used[slot] ? (uint32_t)id : 0u, row_bytes) + col));
     };
 #pragma unroll
     for (int e = 0; e < LD; ++e) request(e, e);
@@ -396,7 +408,7 @@ __global__ __launch_bounds__(kTokensPerBlock* kWave) void expert_split_accumulat
       float sdot = 0.f;
       for (int cb = 0; cb < col_blocks; ++cb) {                  // slice order, column block by column block
 #pragma unroll
-        for (int sl = 0; sl < kSlices; ++sl) sdot += partial[((int64_t(cb) * kSlices + sl) * num_tokens + tt) * top_k + j];
+        for (int sl = 0; sl < kSlices; ++sl) sdot += partial[((Off(cb) * kSlices + sl) * num_tokens + tt) * top_k + j];
       }
       coef = silu_f32(sdot) * Elem<DT>::load(gates, base + j);
     }
@@ -407,7 +419,7 @@ __global__ __launch_bounds__(kTokensPerBlock* kWave) void expert_split_accumulat
       if (e + LD < LPR) request(e % LD, e + LD);
     }
   }
-  if (live) *(u32x4_t*)(y + t * row_bytes + col) = pack16<DT>(acc);
+  if (live) *(u32x4_t*)(y + (split_mul<SMALL>((uint32_t)t, row_bytes) + col)) = pack16<DT>(acc);
 }
 
 // lanes per row slice, or 0 when the row does not cut into 8 slices of 4..64 lanes
@@ -429,23 +441,40 @@ static inline int split_col_blocks(int hidden, int elem_bytes, int* lanes_per_ro
   return 0;
 }
 
-template <int DT, int LPR>
-static hipError_t launch_split(const void* x, const void* up, const void* down, const void* gates, const int32_t* ids,
-                               float* partial, void* y, int64_t T, int H, int k, int64_t N, int col_blocks, hipStream_t s) {
+// every byte offset into x, y, the tables and the partial sums fits 32 bits, and the factors of its products 24
+static inline bool split_offsets_small(int64_t T, int H, int k, int64_t N, int col_blocks, int elem_bytes) {
+  const int64_t row = (int64_t)H * elem_bytes, lim = (int64_t)1 << 32, f24 = (int64_t)1 << 24;
+  return row < f24 && N < f24 && T < f24 && k < f24 && N * row < lim && T * row < lim && T * k < lim &&
+         (int64_t)kSlices * col_blocks * T * k * 4 < lim;
+}
+
+template <int DT, int LPR, bool SMALL>
+static hipError_t launch_split_as(const void* x, const void* up, const void* down, const void* gates, const int32_t* ids,
+                                  float* partial, void* y, int64_t T, int H, int k, int64_t N, int col_blocks, hipStream_t s) {
   constexpr int kPerBlock = kTokensPerBlock * (kWave / LPR);       // tokens per block
+  // measured (bf16, same box): the dots pass gains 1-3 % from 32-bit offsets at every slice length; the accumulate pass gains
+  // 3 % at 512-byte slices and LOSES 4-8 % at 256-byte ones (the compiler's schedule of its row window changes with them)
+  constexpr bool kAccSmall = SMALL && LPR >= 32;
   const unsigned blocks = (unsigned)((T + kPerBlock - 1) / kPerBlock) * kSlices;
   for (int cb = 0; cb < col_blocks; ++cb)                            // all partial dot products first: a coefficient needs the whole row
-    hipLaunchKernelGGL((expert_split_dots_kernel<DT, LPR>), dim3(blocks), dim3(kTokensPerBlock * kWave), 0, s, (const uint8_t*)x,
+    hipLaunchKernelGGL((expert_split_dots_kernel<DT, LPR, SMALL>), dim3(blocks), dim3(kTokensPerBlock * kWave), 0, s, (const uint8_t*)x,
                        (const uint8_t*)up, ids, partial, (int)T, H, k, (uint32_t)N, cb);
   if (col_blocks == 1) {
-    hipLaunchKernelGGL((expert_split_accumulate_kernel<DT, LPR, false>), dim3(blocks), dim3(kTokensPerBlock * kWave), 0, s,
+    hipLaunchKernelGGL((expert_split_accumulate_kernel<DT, LPR, false, kAccSmall>), dim3(blocks), dim3(kTokensPerBlock * kWave), 0, s,
                        (const uint8_t*)down, gates, ids, partial, (uint8_t*)y, (int)T, H, k, (uint32_t)N, 0, 1);
     return hipGetLastError();
   }
   for (int cb = 0; cb < col_blocks; ++cb)
-    hipLaunchKernelGGL((expert_split_accumulate_kernel<DT, LPR, true>), dim3(blocks), dim3(kTokensPerBlock * kWave), 0, s,
+    hipLaunchKernelGGL((expert_split_accumulate_kernel<DT, LPR, true, kAccSmall>), dim3(blocks), dim3(kTokensPerBlock * kWave), 0, s,
                        (const uint8_t*)down, gates, ids, partial, (uint8_t*)y, (int)T, H, k, (uint32_t)N, cb, col_blocks);
   return hipGetLastError();
+}
+template <int DT, int LPR>
+static hipError_t launch_split(const void* x, const void* up, const void* down, const void* gates, const int32_t* ids,
+                               float* partial, void* y, int64_t T, int H, int k, int64_t N, int col_blocks, hipStream_t s) {
+  if (split_offsets_small(T, H, k, N, col_blocks, DT == kF32 ? 4 : 2))
+    return launch_split_as<DT, LPR, true>(x, up, down, gates, ids, partial, y, T, H, k, N, col_blocks, s);
+  return launch_split_as<DT, LPR, false>(x, up, down, gates, ids, partial, y, T, H, k, N, col_blocks, s);
 }
 
 // workspace: partial dot products [8 * column blocks][T][k] f32

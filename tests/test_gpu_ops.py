@@ -275,6 +275,32 @@ def test_expert_split_algorithm(case, device):
     assert (got.float() - ref).abs().max().item() <= (1e-2 if dtype != torch.float32 else 1e-5) * scale
 
 
+def test_expert_split_tables_beyond_4gib(device):
+    """Tables of 4 GiB each: the split kernels then take their 64-bit row offsets (below that size they use 32-bit ones).
+    Rows built on the device, ids from both ends of the tables; checked against the oracle on the rows that are used."""
+    T, H, N, k = 256, 2048, 1 << 20, 8
+    g = torch.Generator().manual_seed(11)
+    print(f"expert split 4 GiB tables T={T} H={H} N={N} k={k}", flush=True)
+    up = torch.empty(N, H, dtype=torch.bfloat16, device=device).normal_(0, 0.05)
+    down = torch.empty(N, H, dtype=torch.bfloat16, device=device).normal_(0, 0.05)
+    x = (torch.randn(T, H, generator=g) * 0.5).bfloat16()
+    gates = torch.rand(T, k, generator=g).bfloat16()
+    ids = torch.randint(0, N, (T, k), generator=g, dtype=torch.int32)
+    ids[:, 0] = N - 1 - torch.arange(T, dtype=torch.int32)            # the far end: byte offsets beyond 2^32
+    ids[:, 1] = torch.arange(T, dtype=torch.int32)
+    d = [x.to(device), up, down, gates.to(device), ids.to(device)]
+    got = _ops().hip_omni_expert_func(*d, algo="split")
+    ref = _ops().hip_omni_expert_func(*d, algo="gather")
+    # the oracle on a compact copy of the rows in use
+    used, inv = torch.unique(ids.long(), return_inverse=True)
+    want = oracle.expert_forward(x, up[used.to(device)].cpu(), down[used.to(device)].cpu(), gates, inv.int())
+    torch.testing.assert_close(got.cpu().float(), want.float(), **_tol(torch.bfloat16))
+    scale = max(ref.float().abs().max().item(), 1e-6)
+    assert (got.float() - ref.float()).abs().max().item() <= 1e-2 * scale
+    del up, down
+    torch.cuda.empty_cache()
+
+
 DENSE_CASES = [(16384, 1024, 256, 16, torch.bfloat16, "baseline"),   # the shape the build plan names for the group regime: 1024 pairs per expert
                (4096, 512, 64, 8, torch.bfloat16, "ref"),              # negative gates, ids with replacement (duplicates add)
                (2048, 256, 32, 6, torch.float16, "ref"),
