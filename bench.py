@@ -46,9 +46,9 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 # Bytes that cross the fabric per launch (FETCH_SIZE + WRITE_SIZE of rocprofv3 --pmc, each scaled by a plain copy of
 # known size); counters cannot be read in-process, so these are the figures of the committed summaries named here.
 TRAFFIC_SOURCE = ("profiles/bench_layer_c4_hbm_counters.txt, profiles/expert_c5_hbm_counters.txt; measured on the kernels as of the commit "
-                  "'Streaming GEMM: scalar work per K tile cut' -- a later change to a kernel's memory access pattern needs a new counter run")
-TRAFFIC_BYTES = {"expert_c3": 180.6e6, "expert_c4": 57.8e6, "expert_gather_c3": 899.4e6, "gateup_c4": 134.4e6, "down_c4": 117.6e6,
-                 "down_plain_c4": 109.2e6, "schedule_c3": 12.36e6, "expert_segment_c3": 928.1e6, "expert_bwd_c3": 2159.8e6,
+                  "'Expert split passes: 32-bit row offsets' -- a later change to a kernel's memory access pattern needs a new counter run")
+TRAFFIC_BYTES = {"expert_c3": 180.6e6, "expert_c4": 57.8e6, "expert_gather_c3": 900.0e6, "gateup_c4": 134.4e6, "down_c4": 117.6e6,
+                 "down_plain_c4": 109.2e6, "schedule_c3": 12.36e6, "expert_segment_c3": 928.1e6, "expert_bwd_c3": 2160.2e6,
                  "expert_c5_routed": 1029.1e6, "expert_c5_routed_split": 724.9e6, "expert_c5_uniform": 8848.6e6}
 SECTIONS = ("layer", "kernels", "expert_c3", "expert_c5", "layer_c5", "ref_grid", "probe", "train", "cpu")
 
